@@ -1,0 +1,104 @@
+// C ABI of libflashcolsum.so: argument checks, launch plan, workspace carving.
+// Declarations and the reference call sites they replace: include/flash_colsum.h.
+#include <math.h>
+#include <string.h>
+
+#include "flash_colsum.h"
+#include "fcs_kernels.h"
+
+namespace {
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// last-dim stride 1 and every other stride a multiple of 8 halves (16 bytes)
+bool strides_ok(const int64_t s[4], bool use_batch)
+{
+    if (s[3] != 1) return false;
+    if ((s[2] & 7) || (s[1] & 7)) return false;
+    if (use_batch && (s[0] & 7)) return false;
+    return true;
+}
+
+int run(int causal, const void *q, const void *k, float *out, void *ws, size_t ws_bytes, int B, int H,
+        int Sq, int Sk, int D, const int64_t qs[4], const int64_t ks[4], float scale, int cls_n,
+        int k_past, void *stream)
+{
+    if (!q || !k || !out || !qs || !ks) return FCS_E_NULL;
+    if (B < 1 || H < 1 || Sq < 1 || Sk < 1 || D < 1 || cls_n == 0 || k_past < 0) return FCS_E_DIMS;
+    if ((long)B * H > 65535) return FCS_E_DIMS;
+    if (D != 64 && D != 128) return FCS_E_HEAD_DIM;
+    if (!strides_ok(qs, B > 1) || !strides_ok(ks, B > 1) || !aligned16(q) || !aligned16(k)) return FCS_E_STRIDE;
+    if (!isfinite(scale)) return FCS_E_SCALE;
+
+    fcs::Plan p;
+    if (!fcs::make_plan(p, causal, B, H, Sq, Sk, D, cls_n, k_past)) return FCS_E_DIMS;
+    if (p.total > 0 && (!ws || ws_bytes < p.total)) return ws ? FCS_E_WORKSPACE : FCS_E_NULL;
+
+    fcs::Args a;
+    memset(&a, 0, sizeof(a));
+    a.q = static_cast<const _Float16 *>(q);
+    a.k = static_cast<const _Float16 *>(k);
+    a.qs_b = qs[0]; a.qs_h = qs[1]; a.qs_s = qs[2];
+    a.ks_b = ks[0]; a.ks_h = ks[1]; a.ks_s = ks[2];
+    a.B = B; a.H = H; a.Sq = Sq; a.Sk = Sk;
+    a.q_rows = p.q_rows;
+    a.causal = p.causal; a.k_past = p.k_past;
+    a.negate = scale < 0.f;
+    a.c = fabsf(scale) * 1.44269504088896340736f;
+    a.n_chunks = p.n_chunks; a.chunk_keys = p.chunk_keys; a.rows_pad = p.rows_pad;
+    char *w = static_cast<char *>(ws);
+    a.lse = reinterpret_cast<float *>(w + p.off_lse);
+    a.ml = reinterpret_cast<float2 *>(w + p.off_ml);
+    a.gh = p.gh; a.gq = p.gq;
+    a.heads_per_group = p.heads_per_group; a.qtiles_per_group = p.qtiles_per_group;
+    a.partial = reinterpret_cast<float *>(w + p.off_partial);
+    a.out = out;
+    a.inv_norm = 1.0f / ((float)H * (float)p.q_rows);
+    return fcs::launch_colsum(p, a, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+int fcs_abi_version(void) { return FCS_ABI_VERSION; }
+
+const char *fcs_strerror(int code)
+{
+    switch (code) {
+    case FCS_OK: return "ok";
+    case FCS_E_NULL: return "a required pointer is NULL";
+    case FCS_E_DIMS: return "invalid dimension (each of B,H,S,D must be >= 1, B*H <= 65535, cls_n != 0, k_past >= 0)";
+    case FCS_E_HEAD_DIM: return "unsupported head dim (compiled: 64, 128)";
+    case FCS_E_STRIDE: return "unsupported layout (last stride must be 1; rows, heads and base 16-byte aligned)";
+    case FCS_E_WORKSPACE: return "workspace smaller than fcs_workspace_bytes()";
+    case FCS_E_SCALE: return "scale is not finite";
+    default: return code > 0 ? "HIP launch error (code is a hipError_t)" : "unknown error code";
+    }
+}
+
+size_t fcs_workspace_bytes(int causal, int B, int H, int Sq, int Sk, int D, int cls_n)
+{
+    fcs::Plan p;
+    const int k_past = (causal && Sk > Sq) ? Sk - Sq : 0;  // the layout does not depend on k_past
+    if (!fcs::make_plan(p, causal, B, H, Sq, Sk, D, cls_n, k_past)) return 0;
+    return p.total;
+}
+
+int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *ws, size_t ws_bytes, int B, int H,
+                             int S, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
+                             int cls_n, void *hip_stream)
+{
+    return run(0, q, k, out, ws, ws_bytes, B, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
+               hip_stream);
+}
+
+int fcs_colsum_causal_f16(const void *q, const void *k, float *out, void *ws, size_t ws_bytes, int H, int Q_len,
+                          int K_len, int D, int k_past, const int64_t q_strides[4], const int64_t k_strides[4],
+                          float scale, void *hip_stream)
+{
+    return run(1, q, k, out, ws, ws_bytes, 1, H, Q_len, K_len, D, q_strides, k_strides, scale, -1, k_past,
+               hip_stream);
+}
+
+}  // extern "C"

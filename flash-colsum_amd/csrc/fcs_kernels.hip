@@ -1,0 +1,419 @@
+// Attention column means on gfx950 (MI355X): the general two-pass path.
+//
+// Both passes compute 32x32 score tiles  S^T = K_tile * Q_tile^T  on
+// v_mfma_f32_32x32x16_f16, so that a lane owns ONE query (column l%32 of the tile) and
+// holds 16 keys of it in its accumulator registers (key row 8*(r/4) + 4*(l/32) + r%4).
+//
+//   pass 1 (fcs_rowstats_kernel)  Q tile stationary in registers, K streamed through LDS.
+//          Row max and sum-of-exp are then plain in-lane running scalars; the two
+//          half-waves are combined once at the end.  Emits lse2[i] = log2 sum_j 2^(c*s_ij)
+//          (c = scale*log2(e)), or a partial (max,sum) per key split.
+//   pass 2 (fcs_colsum_kernel)    K tile stationary in registers, Q (+ lse2) streamed
+//          through LDS.  p_ij = 2^(c*s_ij - lse2[i]) is one FMA and one v_exp_f32; each
+//          lane adds it into a per-key register, and the 32 query lanes are summed once
+//          at the very end.  No atomics: every partial has exactly one writer and the
+//          groups are added in a fixed order by fcs_finalize_kernel.
+//
+// The fragment <-> head-dim mapping (which 8 channels a lane feeds to which MFMA step) is
+// the same for both operands, which is all the contraction needs.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fcs_kernels.h"
+
+namespace fcs {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+static constexpr float kNegBig = -1.0e30f;  // "hidden" score: finite so that max/sub never make NaN
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+__device__ __forceinline__ half8 load8(const _Float16 *p) { return *reinterpret_cast<const half8 *>(p); }
+
+__device__ __forceinline__ half8 flip_sign(half8 v)
+{
+    uint4v u = __builtin_bit_cast(uint4v, v);
+    u ^= 0x80008000u;
+    return __builtin_bit_cast(half8, u);
+}
+
+// key (A-operand row) held by accumulator register i of a lane in half-wave g
+__device__ __forceinline__ int acc_row(int i, int g) { return 8 * (i >> 2) + 4 * g + (i & 3); }
+
+// ------------------------------------------------------------------------------------
+// pass 1: per-row log-sum-exp (or per-split partials)
+// ------------------------------------------------------------------------------------
+template <int D, int QW>
+__global__ __launch_bounds__(256, 2) void fcs_rowstats_kernel(const Args a)
+{
+    constexpr int NB = QW / 32;         // query fragments per wave
+    constexpr int NT = D / 16;          // MFMA steps along the head dim
+    constexpr int KT = kStageKeys;      // keys per LDS stage
+    constexpr int NA = KT / 32;         // key fragments per stage
+    constexpr int PITCH = D + 8;        // halves per LDS row (+16 B: conflict-free b128 reads)
+    constexpr int CPR = D / 8;          // 16-byte pieces per row
+    constexpr int CPT = KT * CPR / 256; // pieces per thread per stage
+    __shared__ __attribute__((aligned(16))) _Float16 lds[2][KT * PITCH];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
+    const int bh = blockIdx.z, b = bh / a.H, h = bh - b * a.H;
+    const int chunk = blockIdx.y;
+    const int q0 = blockIdx.x * (4 * QW);
+    const int qw0 = q0 + wave * QW;
+    const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
+    const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)h * a.ks_h;
+
+    // key range of this block: its split, cut at the last key any of its rows may see
+    const int kc0 = chunk * a.chunk_keys;
+    int kc1 = min(a.Sk, kc0 + a.chunk_keys);
+    if (a.causal) kc1 = min(kc1, a.k_past + min(q0 + 4 * QW, a.q_rows));
+    const int nst = (kc1 > kc0) ? (kc1 - kc0 + KT - 1) / KT : 0;
+
+    half8 qf[NB][NT];
+    int thr[NB];  // last visible key of the lane's query
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int qi = qw0 + nb * 32 + r;
+        const _Float16 *row = qp + (int64_t)min(qi, a.Sq - 1) * a.qs_s + g * 8;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            half8 v = load8(row + t * 16);
+            qf[nb][t] = a.negate ? flip_sign(v) : v;
+        }
+        thr[nb] = a.causal ? min(a.k_past + qi, a.Sk - 1) : a.Sk - 1;
+    }
+    const int thr_min = a.causal ? min(a.k_past + qw0, a.Sk - 1) : a.Sk - 1;  // wave-uniform
+
+    float m[NB], l[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) { m[nb] = kNegBig; l[nb] = 0.f; }
+
+    half8 stg[CPT];
+    auto gload = [&](int kb) {
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int c = tid + i * 256, row = c / CPR, col = (c % CPR) * 8;
+            stg[i] = load8(kp + (int64_t)min(kb + row, a.Sk - 1) * a.ks_s + col);
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int c = tid + i * 256, row = c / CPR, col = (c % CPR) * 8;
+            *reinterpret_cast<half8 *>(&lds[buf][row * PITCH + col]) = stg[i];
+        }
+    };
+
+    if (nst > 0) { gload(kc0); lstore(0); }
+    __syncthreads();
+    for (int it = 0; it < nst; ++it) {
+        const int kb = kc0 + it * KT;
+        if (it + 1 < nst) gload(kb + KT);
+        const _Float16 *tile = lds[it & 1];
+
+        floatx16 acc[NA][NB];
+#pragma unroll
+        for (int na = 0; na < NA; ++na) {
+            half8 af[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                af[t] = *reinterpret_cast<const half8 *>(&tile[(na * 32 + r) * PITCH + t * 16 + g * 8]);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t], qf[nb][t], c, 0, 0, 0);
+                acc[na][nb] = c;
+            }
+        }
+
+        const bool edge = (kb + KT - 1 > thr_min);  // stage holds keys hidden from some row of this wave
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            if (!edge) {
+                float tmax = acc[0][nb][0];
+#pragma unroll
+                for (int na = 0; na < NA; ++na)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, acc[na][nb][i]);
+                const float mn = fmaxf(m[nb], tmax);
+                const float alpha = fast_exp2((m[nb] - mn) * a.c);
+                const float nm = -mn * a.c;
+                float sum = 0.f;
+#pragma unroll
+                for (int na = 0; na < NA; ++na)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) sum += fast_exp2(fmaf(acc[na][nb][i], a.c, nm));
+                l[nb] = l[nb] * alpha + sum;
+                m[nb] = mn;
+            } else {
+                float tmax = kNegBig;
+#pragma unroll
+                for (int na = 0; na < NA; ++na)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const bool vis = (kb + na * 32 + acc_row(i, g)) <= thr[nb];
+                        tmax = fmaxf(tmax, vis ? acc[na][nb][i] : kNegBig);
+                    }
+                const float mn = fmaxf(m[nb], tmax);
+                const float alpha = fast_exp2((m[nb] - mn) * a.c);
+                const float nm = -mn * a.c;
+                float sum = 0.f;
+#pragma unroll
+                for (int na = 0; na < NA; ++na)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const bool vis = (kb + na * 32 + acc_row(i, g)) <= thr[nb];
+                        const float e = fast_exp2(fmaf(acc[na][nb][i], a.c, nm));
+                        sum += vis ? e : 0.f;
+                    }
+                l[nb] = l[nb] * alpha + sum;
+                m[nb] = mn;
+            }
+        }
+
+        if (it + 1 < nst) lstore((it + 1) & 1);
+        __syncthreads();
+    }
+
+    // combine the two half-waves (same query, disjoint keys) and store
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const float m2 = __shfl_xor(m[nb], 32), l2 = __shfl_xor(l[nb], 32);
+        const float mm = fmaxf(m[nb], m2);
+        const float ll = l[nb] * fast_exp2((m[nb] - mm) * a.c) + l2 * fast_exp2((m2 - mm) * a.c);
+        if (g == 0) {
+            const int qi = qw0 + nb * 32 + r;  // < rows_pad by construction
+            if (a.n_chunks == 1) {
+                a.lse[(int64_t)bh * a.rows_pad + qi] = mm * a.c + fast_log2(ll);
+            } else {
+                float2 v;
+                v.x = mm * a.c;
+                v.y = ll;
+                a.ml[((int64_t)bh * a.n_chunks + chunk) * a.rows_pad + qi] = v;
+            }
+        }
+    }
+}
+
+// merge the per-split (max, sum) partials of pass 1 into lse2
+__global__ __launch_bounds__(256) void fcs_merge_stats_kernel(const Args a)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    const int bh = blockIdx.y;
+    if (i >= a.rows_pad) return;
+    const float2 *p = a.ml + (int64_t)bh * a.n_chunks * a.rows_pad + i;
+    float mm = -INFINITY;
+    for (int c = 0; c < a.n_chunks; ++c) mm = fmaxf(mm, p[(int64_t)c * a.rows_pad].x);
+    float ll = 0.f;
+    for (int c = 0; c < a.n_chunks; ++c) {
+        const float2 v = p[(int64_t)c * a.rows_pad];
+        ll += v.y * fast_exp2(v.x - mm);
+    }
+    a.lse[(int64_t)bh * a.rows_pad + i] = mm + fast_log2(ll);
+}
+
+// ------------------------------------------------------------------------------------
+// pass 2: column sums of p_ij = 2^(c*s_ij - lse2[i])
+// ------------------------------------------------------------------------------------
+template <int D, int KW>
+__global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
+{
+    constexpr int NA = KW / 32;
+    constexpr int NT = D / 16;
+    constexpr int QT = kStageRows;
+    constexpr int NB = QT / 32;
+    constexpr int PITCH = D + 8;
+    constexpr int CPR = D / 8;
+    constexpr int CPT = QT * CPR / 256;
+    __shared__ __attribute__((aligned(16))) _Float16 lds[2][QT * PITCH];
+    __shared__ float lse_s[2][QT];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
+    const int b = blockIdx.z;
+    const int grp = blockIdx.y, gh_i = grp / a.gq, gq_i = grp - gh_i * a.gq;
+    const int k0 = blockIdx.x * (4 * KW);
+    const int kw0 = k0 + wave * KW;
+    const int kmax_w = kw0 + KW - 1;
+
+    const int h_begin = gh_i * a.heads_per_group;
+    const int h_end = min(a.H, h_begin + a.heads_per_group);
+    const int n_qt = (a.q_rows + QT - 1) / QT;
+    int t_begin = gq_i * a.qtiles_per_group;
+    const int t_end = min(n_qt, t_begin + a.qtiles_per_group);
+    if (a.causal) t_begin = max(t_begin, max(0, k0 - a.k_past) / QT);  // earlier rows see none of these keys
+    const int nt = max(0, t_end - t_begin);
+    const int nst = nt * max(0, h_end - h_begin);
+
+    floatx16 colacc[NA];
+#pragma unroll
+    for (int na = 0; na < NA; ++na)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) colacc[na][i] = 0.f;
+
+    half8 kf[NA][NT];
+    half8 stg[CPT];
+    float stg_lse = 0.f;
+    auto gload = [&](int s) {
+        const int h = h_begin + s / nt, t = t_begin + s % nt;
+        const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int c = tid + i * 256, row = c / CPR, col = (c % CPR) * 8;
+            stg[i] = load8(qp + (int64_t)min(t * QT + row, a.Sq - 1) * a.qs_s + col);
+        }
+        if (tid < QT) {
+            const int qi = t * QT + tid;
+            stg_lse = (qi < a.q_rows) ? a.lse[((int64_t)b * a.H + h) * a.rows_pad + qi] : INFINITY;
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int c = tid + i * 256, row = c / CPR, col = (c % CPR) * 8;
+            *reinterpret_cast<half8 *>(&lds[buf][row * PITCH + col]) = stg[i];
+        }
+        if (tid < QT) lse_s[buf][tid] = stg_lse;
+    };
+
+    if (nst > 0) { gload(0); lstore(0); }
+    __syncthreads();
+    for (int s = 0; s < nst; ++s) {
+        const int hs = s / nt, t = t_begin + (s - hs * nt);
+        if (s - hs * nt == 0) {  // new head: fetch this wave's key fragments
+            const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)(h_begin + hs) * a.ks_h;
+#pragma unroll
+            for (int na = 0; na < NA; ++na) {
+                const _Float16 *row = kp + (int64_t)min(kw0 + na * 32 + r, a.Sk - 1) * a.ks_s + g * 8;
+#pragma unroll
+                for (int tt = 0; tt < NT; ++tt) {
+                    half8 v = load8(row + tt * 16);
+                    kf[na][tt] = a.negate ? flip_sign(v) : v;
+                }
+            }
+        }
+        if (s + 1 < nst) gload(s + 1);
+        const _Float16 *tile = lds[s & 1];
+
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            half8 bf[NT];
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt)
+                bf[tt] = *reinterpret_cast<const half8 *>(&tile[(nb * 32 + r) * PITCH + tt * 16 + g * 8]);
+            const float nlse = -lse_s[s & 1][nb * 32 + r];
+            const int qmin = t * QT + nb * 32;
+            const bool edge = a.causal && (kmax_w > a.k_past + qmin);  // wave-uniform
+#pragma unroll
+            for (int na = 0; na < NA; ++na) {
+                floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int tt = 0; tt < NT; ++tt)
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[na][tt], bf[tt], c, 0, 0, 0);
+                if (!edge) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) colacc[na][i] += fast_exp2(fmaf(c[i], a.c, nlse));
+                } else {
+                    const int lim = a.k_past + qmin + r;  // last key this lane's query sees
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const float p = fast_exp2(fmaf(c[i], a.c, nlse));
+                        colacc[na][i] += (kw0 + na * 32 + acc_row(i, g) <= lim) ? p : 0.f;
+                    }
+                }
+            }
+        }
+
+        if (s + 1 < nst) lstore((s + 1) & 1);
+        __syncthreads();
+    }
+
+    // sum the 32 query lanes of each half-wave; lane r == 0 of each half writes its 16 keys
+    const bool direct = (a.gh * a.gq == 1);
+#pragma unroll
+    for (int na = 0; na < NA; ++na) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float v = colacc[na][i];
+            v += __shfl_xor(v, 16);
+            v += __shfl_xor(v, 8);
+            v += __shfl_xor(v, 4);
+            v += __shfl_xor(v, 2);
+            v += __shfl_xor(v, 1);
+            const int key = kw0 + na * 32 + acc_row(i, g);
+            if (r == 0 && key < a.Sk) {
+                if (direct)
+                    a.out[(int64_t)b * a.Sk + key] = v * a.inv_norm;
+                else
+                    a.partial[((int64_t)grp * a.B + b) * a.Sk + key] = v;
+            }
+        }
+    }
+}
+
+// out = inv_norm * (partial[0] + partial[1] + ...), groups added in index order
+__global__ __launch_bounds__(256) void fcs_finalize_kernel(const Args a)
+{
+    const int64_t n = (int64_t)a.B * a.Sk;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int ng = a.gh * a.gq;
+    float s = 0.f;
+    for (int gi = 0; gi < ng; ++gi) s += a.partial[(int64_t)gi * n + idx];
+    a.out[idx] = s * a.inv_norm;
+}
+
+// ------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------
+template <int D>
+static hipError_t launch_d(const Plan &p, const Args &a, hipStream_t st)
+{
+    const dim3 blk(256);
+    {
+        const dim3 grid(p.n_qblk, p.n_chunks, p.B * p.H);
+        if (p.qw == 64)
+            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64>), grid, blk, 0, st, a);
+        else
+            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 32>), grid, blk, 0, st, a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (p.n_chunks > 1) {
+        const dim3 grid((p.rows_pad + 255) / 256, p.B * p.H);
+        hipLaunchKernelGGL(fcs_merge_stats_kernel, grid, blk, 0, st, a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    {
+        const dim3 grid(p.n_kblk, p.gh * p.gq, p.B);
+        if (p.kw == 64)
+            hipLaunchKernelGGL((fcs_colsum_kernel<D, 64>), grid, blk, 0, st, a);
+        else
+            hipLaunchKernelGGL((fcs_colsum_kernel<D, 32>), grid, blk, 0, st, a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (p.gh * p.gq > 1) {
+        const int64_t n = (int64_t)p.B * p.Sk;
+        const dim3 grid((unsigned)((n + 255) / 256));
+        hipLaunchKernelGGL(fcs_finalize_kernel, grid, blk, 0, st, a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+int launch_colsum(const Plan &p, const Args &a, void *stream)
+{
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    hipError_t e = (p.D == 64) ? launch_d<64>(p, a, st) : launch_d<128>(p, a, st);
+    return (int)e;
+}
+
+}  // namespace fcs

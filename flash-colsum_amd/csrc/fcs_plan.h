@@ -1,0 +1,91 @@
+// Launch plan for the column-mean kernels: how one call is cut into workgroups and how
+// the caller's workspace is laid out.  Pure host arithmetic, shared by
+// fcs_workspace_bytes() and the launch functions so both always agree.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+namespace fcs {
+
+constexpr int kWavesPerBlock = 4;   // 256 threads
+constexpr int kStageKeys = 64;      // keys staged in LDS per step of the row-statistics pass
+constexpr int kStageRows = 64;      // query rows staged in LDS per step of the column pass
+constexpr int kTargetBlocks = 1024; // 256 CUs x 4: enough workgroups to fill the chip twice over
+
+struct Plan {
+    int B, H, Sq, Sk, D;
+    int q_rows;  // query rows that are averaged: min(cls_n, Sq) or Sq
+    int causal, k_past;
+    // pass 1: row statistics.  grid = (n_qblk, n_chunks, B*H)
+    int qw;          // query rows per wave (32 or 64); a block covers 4*qw rows
+    int n_qblk;      // blocks along the query axis
+    int n_chunks;    // key-axis splits (partial (max,sum) per chunk when > 1)
+    int chunk_keys;  // keys per split, multiple of kStageKeys
+    int rows_pad;    // n_qblk * 4 * qw  (row pitch of the statistics arrays)
+    // pass 2: column sums.  grid = (n_kblk, gh*gq, B)
+    int kw;          // keys per wave (32 or 64); a block covers 4*kw keys
+    int n_kblk;
+    int gh, gq;      // groups along heads / along staged query tiles
+    int heads_per_group, qtiles_per_group;
+    // workspace layout (byte offsets, each 256-byte aligned)
+    size_t off_lse;      // float  [B*H][rows_pad]            log2-domain log-sum-exp
+    size_t off_ml;       // float2 [B*H][n_chunks][rows_pad]  only when n_chunks > 1
+    size_t off_partial;  // float  [gh*gq][B][Sk]             only when gh*gq > 1
+    size_t total;
+};
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// Returns false for invalid dimensions.  cls_n <= 0 means all rows.
+inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, int cls_n, int k_past)
+{
+    if (B < 1 || H < 1 || Sq < 1 || Sk < 1 || D < 1 || k_past < 0) return false;
+    p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk; p.D = D;
+    p.causal = causal ? 1 : 0;
+    p.k_past = causal ? k_past : 0;
+    p.q_rows = (!causal && cls_n > 0 && cls_n < Sq) ? cls_n : Sq;
+
+    // ---- pass 1
+    p.qw = (p.q_rows > 128) ? 64 : 32;
+    const int qblk = kWavesPerBlock * p.qw;
+    p.n_qblk = ceil_div(p.q_rows, qblk);
+    p.rows_pad = p.n_qblk * qblk;
+    const long base1 = (long)p.n_qblk * B * H;
+    int want = (int)((kTargetBlocks + base1 - 1) / base1);
+    int max_chunks = ceil_div(Sk, 4 * kStageKeys);  // at least 256 keys per split
+    if (want > max_chunks) want = max_chunks;
+    if (want < 1) want = 1;
+    p.chunk_keys = ceil_div(ceil_div(Sk, want), kStageKeys) * kStageKeys;
+    p.n_chunks = ceil_div(Sk, p.chunk_keys);
+
+    // ---- pass 2
+    const int n_qt = ceil_div(p.q_rows, kStageRows);
+    p.kw = ((long)ceil_div(Sk, 256) * B >= kTargetBlocks / 4) ? 64 : 32;
+    const int kblk = kWavesPerBlock * p.kw;
+    p.n_kblk = ceil_div(Sk, kblk);
+    const long base2 = (long)p.n_kblk * B;
+    int g = (int)((kTargetBlocks + base2 - 1) / base2);
+    if (g < 1) g = 1;
+    p.gh = g < H ? g : H;
+    p.heads_per_group = ceil_div(H, p.gh);
+    p.gh = ceil_div(H, p.heads_per_group);
+    int gq = ceil_div(g, p.gh);
+    if (gq > n_qt) gq = n_qt;
+    if (gq < 1) gq = 1;
+    p.qtiles_per_group = ceil_div(n_qt, gq);
+    p.gq = ceil_div(n_qt, p.qtiles_per_group);
+
+    // ---- workspace
+    size_t off = 0;
+    p.off_lse = off;
+    off = align256(off + sizeof(float) * (size_t)B * H * p.rows_pad);
+    p.off_ml = off;
+    if (p.n_chunks > 1) off = align256(off + 2 * sizeof(float) * (size_t)B * H * p.n_chunks * p.rows_pad);
+    p.off_partial = off;
+    if (p.gh * p.gq > 1) off = align256(off + sizeof(float) * (size_t)p.gh * p.gq * B * Sk);
+    p.total = off;
+    return true;
+}
+
+}  // namespace fcs

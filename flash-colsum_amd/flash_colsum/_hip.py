@@ -1,0 +1,133 @@
+"""Host layer: binds libflashcolsum.so (C ABI, include/flash_colsum.h) with ctypes.
+
+PyTorch supplies device memory and the HIP stream; every byte of arithmetic happens in
+the hand-written gfx950 kernels behind the C ABI.  There is no fallback: if the shared
+library is missing or a launch fails this module raises.
+
+The three private launchers keep the names and argument meaning of the reference's
+(reference: flash_colsum/kernel_noncausal_batched.py:102, kernel_noncausal.py:95,
+kernel_causal.py:94) and, like them, return fp16; the `*_f32` functions return the
+kernels' fp32 means.
+"""
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libflashcolsum.so")
+_ABI_VERSION = 1
+_lib = None
+
+_I64x4 = ctypes.c_int64 * 4
+
+
+def lib() -> ctypes.CDLL:
+    """Load the shared library once; raise loudly when it is absent or of another ABI."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                f"{_LIB_PATH} not found: build it with `make -C flash-colsum_amd` "
+                "(hipcc, --offload-arch=gfx950). There is no fallback path."
+            )
+        cdll = ctypes.CDLL(_LIB_PATH)
+        cdll.fcs_abi_version.restype = ctypes.c_int
+        cdll.fcs_abi_version.argtypes = []
+        cdll.fcs_strerror.restype = ctypes.c_char_p
+        cdll.fcs_strerror.argtypes = [ctypes.c_int]
+        cdll.fcs_workspace_bytes.restype = ctypes.c_size_t
+        cdll.fcs_workspace_bytes.argtypes = [ctypes.c_int] * 7
+        cdll.fcs_colsum_noncausal_f16.restype = ctypes.c_int
+        cdll.fcs_colsum_noncausal_f16.argtypes = [
+            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+            ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+            ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
+            ctypes.c_float, ctypes.c_int, ctypes.c_void_p]
+        cdll.fcs_colsum_causal_f16.restype = ctypes.c_int
+        cdll.fcs_colsum_causal_f16.argtypes = [
+            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+            ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+            ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
+            ctypes.c_float, ctypes.c_void_p]
+        got = cdll.fcs_abi_version()
+        if got != _ABI_VERSION:
+            raise RuntimeError(f"libflashcolsum.so has ABI {got}, this host layer needs {_ABI_VERSION}")
+        _lib = cdll
+    return _lib
+
+
+def strerror(code: int) -> str:
+    return lib().fcs_strerror(int(code)).decode()
+
+
+def _check(code: int, what: str) -> None:
+    if code != 0:
+        raise RuntimeError(f"{what} failed with code {code}: {strerror(code)}")
+
+
+def _as_kernel_input(t: torch.Tensor) -> torch.Tensor:
+    """fp16, unit last stride, 16-byte aligned rows/heads/base; copies only when it must."""
+    if t.dtype != torch.float16:
+        t = t.to(torch.float16)
+    ok = (
+        t.stride(3) == 1
+        and t.stride(2) % 8 == 0
+        and t.stride(1) % 8 == 0
+        and (t.shape[0] == 1 or t.stride(0) % 8 == 0)
+        and t.data_ptr() % 16 == 0
+    )
+    return t if ok else t.contiguous()
+
+
+def workspace_bytes(causal: bool, b: int, h: int, s_q: int, s_k: int, d: int, cls_n: int = -1) -> int:
+    return int(lib().fcs_workspace_bytes(int(causal), b, h, s_q, s_k, d, cls_n))
+
+
+def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n: int, k_past: int) -> torch.Tensor:
+    if q.device.type != "cuda" or k.device != q.device:
+        raise ValueError(f"query and key must live on the same GPU, got {q.device} and {k.device}")
+    q = _as_kernel_input(q)
+    k = _as_kernel_input(k)
+    b, h, s_q, d = q.shape
+    s_k = k.shape[2]
+    with torch.cuda.device(q.device):
+        out = torch.empty((b, s_k), dtype=torch.float32, device=q.device)
+        n_ws = workspace_bytes(causal, b, h, s_q, s_k, d, cls_n)
+        ws = torch.empty((max(n_ws, 1),), dtype=torch.uint8, device=q.device)
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        qs, ks = _I64x4(*q.stride()), _I64x4(*k.stride())
+        if causal:
+            rc = lib().fcs_colsum_causal_f16(
+                q.data_ptr(), k.data_ptr(), out.data_ptr(), ws.data_ptr(), n_ws,
+                h, s_q, s_k, d, int(k_past), qs, ks, float(scale), stream)
+        else:
+            rc = lib().fcs_colsum_noncausal_f16(
+                q.data_ptr(), k.data_ptr(), out.data_ptr(), ws.data_ptr(), n_ws,
+                b, h, s_q, d, qs, ks, float(scale), int(cls_n), stream)
+    _check(rc, "fcs_colsum_causal_f16" if causal else "fcs_colsum_noncausal_f16")
+    return out
+
+
+def colsum_noncausal_f32(Q: torch.Tensor, K: torch.Tensor, scale: float, CLS_N: int = -1) -> torch.Tensor:
+    """(B, S) fp32 means over heads and the first min(CLS_N, S) rows (all rows if CLS_N < 0)."""
+    return _launch(False, Q, K, scale, -1 if CLS_N is None or CLS_N < 0 else int(CLS_N), 0)
+
+
+def colsum_causal_f32(Q: torch.Tensor, K: torch.Tensor, scale: float, K_past: Optional[int] = None) -> torch.Tensor:
+    """(1, K_len) fp32 means; K_past defaults to max(0, K_len - Q_len) (reference: kernel_causal.py:113)."""
+    if K_past is None:
+        K_past = max(0, K.shape[2] - Q.shape[2])
+    return _launch(True, Q, K, scale, -1, int(K_past))
+
+
+def _flash_colsum_batched(Q, K, scale, CLS_N=-1):
+    return colsum_noncausal_f32(Q, K, scale, CLS_N).to(torch.float16)
+
+
+def _flash_colsum_non_batched(Q, K, scale, CLS_N=-1):
+    return colsum_noncausal_f32(Q, K, scale, CLS_N).to(torch.float16)
+
+
+def _flash_colsum_causal(Q, K, scale, K_past=None):
+    return colsum_causal_f32(Q, K, scale, K_past).to(torch.float16)

@@ -1,0 +1,81 @@
+"""Public operator: attention column means without the attention matrix.
+
+Drop-in for the reference's `flash_colsum` (reference: flash_colsum/ops.py:13-105): same
+signature, same validation order and `ValueError`s, same result shapes and fp16 result
+dtype.  The three Triton launchers it dispatched to are replaced by the gfx950 HIP
+library bound in `_hip.py`.
+"""
+from typing import Optional
+
+import torch
+
+from . import _hip
+
+
+def _validated(query, key, scale, is_causal, cls_len):
+    """Checks in the reference's order (ops.py:59-97); returns (scale, cls_n)."""
+    if query.ndim != 4 or key.ndim != 4:
+        raise ValueError(f"Expected 4D tensors, got query.ndim={query.ndim}, key.ndim={key.ndim}")
+    if query.device.type != "cuda":
+        raise ValueError(f"flash_colsum only supports CUDA (HIP) tensors, got {query.device}")
+    if cls_len is not None:
+        if is_causal:
+            raise ValueError("cls_len is only supported for non-causal attention")
+        if cls_len <= 0:
+            raise ValueError(f"cls_len must be positive, got {cls_len}")
+    bq, hq, sq, dq = query.shape
+    bk, hk, sk, dk = key.shape
+    if scale is None:
+        scale = dq ** -0.5
+    if is_causal:
+        if bq != 1 or bk != 1:
+            raise ValueError(f"Causal attention currently only supports batch size 1, got B_q={bq}, B_k={bk}")
+        if hq != hk or dq != dk:
+            raise ValueError(
+                f"Query and key must have same heads and head_dim, got H_q={hq}, H_k={hk}, D_q={dq}, D_k={dk}")
+    elif (bq, hq, sq, dq) != (bk, hk, sk, dk):
+        raise ValueError(
+            "For non-causal attention, query and key must have same shape, got "
+            f"query: {tuple(query.shape)}, key: {tuple(key.shape)}")
+    return float(scale), (-1 if cls_len is None else int(cls_len))
+
+
+def flash_colsum_f32(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    scale: Optional[float] = None,
+    is_causal: bool = False,
+    cls_len: Optional[int] = None,
+) -> torch.Tensor:
+    """Same as `flash_colsum` but returns the kernels' fp32 means (no fp16 rounding)."""
+    scale, cls_n = _validated(query, key, scale, is_causal, cls_len)
+    if is_causal:
+        return _hip.colsum_causal_f32(query, key, scale)
+    return _hip.colsum_noncausal_f32(query, key, scale, cls_n)
+
+
+def flash_colsum(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    scale: Optional[float] = None,
+    is_causal: bool = False,
+    cls_len: Optional[int] = None,
+) -> torch.Tensor:
+    """Mean over heads and query rows of softmax(Q K^T * scale), per key position.
+
+    query: (B, H, S, D); for `is_causal` (1, H, Q_len, D).
+    key:   same shape as query; for `is_causal` (1, H, K_len, D), queries aligned to the
+           last Q_len key positions.
+    scale: defaults to 1/sqrt(D).
+    cls_len: non-causal only; average over the first min(cls_len, S) query rows.
+    Returns fp16 (B, S), or (1, K_len) for causal.  Raises ValueError for invalid input.
+    """
+    scale, cls_n = _validated(query, key, scale, is_causal, cls_len)
+    if is_causal:
+        return _hip._flash_colsum_causal(query, key, scale)
+    if query.shape[0] == 1:
+        return _hip._flash_colsum_non_batched(query, key, scale, CLS_N=cls_n)
+    return _hip._flash_colsum_batched(query, key, scale, CLS_N=cls_n)
+
+
+__all__ = ["flash_colsum", "flash_colsum_f32"]

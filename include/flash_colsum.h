@@ -1,0 +1,86 @@
+/* flash_colsum.h -- C ABI of libflashcolsum.so (gfx950 / MI355X).
+ *
+ * Attention column means without materialising the attention matrix:
+ *
+ *     out[b][j] = 1/(H*rows) * sum_h sum_{i<rows} softmax_j( scale * <q[b,h,i,:], k[b,h,j,:]> )
+ *
+ * These entry points are what the host layer of the reference operator binds in place of
+ * its three Triton launchers.  All pointers are DEVICE pointers unless stated otherwise.
+ * The library never allocates, frees or synchronises: the caller owns the output and the
+ * workspace, and every kernel is enqueued on the HIP stream passed in.  Calls are
+ * re-entrant (no mutable global state).
+ *
+ * Return value of the launch functions: 0 = all kernels enqueued; negative = argument
+ * error detected on the host before anything touched the GPU (FCS_E_*); positive = the
+ * hipError_t returned by a failed launch.
+ */
+#ifndef FLASH_COLSUM_H
+#define FLASH_COLSUM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FCS_ABI_VERSION 1
+
+enum {
+    FCS_OK = 0,
+    FCS_E_NULL = -1,      /* a required pointer is NULL                                  */
+    FCS_E_DIMS = -2,      /* a dimension is < 1, or cls_n == 0, or k_past < 0            */
+    FCS_E_HEAD_DIM = -3,  /* D is not one of the compiled head dims (64, 128)            */
+    FCS_E_STRIDE = -4,    /* last-dim stride != 1, or a stride / base not 16-B aligned   */
+    FCS_E_WORKSPACE = -5, /* ws_bytes smaller than fcs_workspace_bytes() for these dims  */
+    FCS_E_SCALE = -6      /* scale is NaN or infinite                                    */
+};
+
+/* ABI version of the loaded library (== FCS_ABI_VERSION of the header it was built with). */
+int fcs_abi_version(void);
+
+/* Static, human-readable text for a return code of this library (negative codes) or a
+ * generic text for positive (HIP) codes.  Never NULL. */
+const char *fcs_strerror(int code);
+
+/* Bytes of device workspace the launch functions need for these dimensions (row
+ * statistics and per-group partial column sums).  `causal` selects the entry point;
+ * for the causal entry point pass B = 1.  `cls_n` <= 0 means "all rows".  Returns 0 for
+ * invalid dimensions.  The workspace needs no initialisation and 256-byte alignment.
+ * Replaces the implicit `torch.zeros` accumulator of the reference launchers
+ * (reference: flash_colsum/kernel_noncausal_batched.py:104, kernel_noncausal.py:98,
+ * kernel_causal.py:105). */
+size_t fcs_workspace_bytes(int causal, int B, int H, int Sq, int Sk, int D, int cls_n);
+
+/* Non-causal column means, fp16 inputs, fp32 output.
+ *   q, k       (B,H,S,D) fp16, element strides q_strides[4] / k_strides[4] (HOST arrays);
+ *              the last stride must be 1 and rows must be 16-byte aligned.
+ *   out        (B,S) fp32 contiguous; receives the MEANS (already divided by H*rows).
+ *   cls_n      <= -1 (or any negative): average over all S query rows;
+ *              >= 1: average over the first min(cls_n, S) query rows only.
+ * Replaces `_flash_colsum_batched(Q, K, scale, CLS_N)` and
+ * `_flash_colsum_non_batched(Q, K, scale, CLS_N)` including their host epilogue
+ * (reference: flash_colsum/kernel_noncausal_batched.py:102-125,
+ * flash_colsum/kernel_noncausal.py:95-117; called from flash_colsum/ops.py:102-105). */
+int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *ws, size_t ws_bytes,
+                             int B, int H, int S, int D,
+                             const int64_t q_strides[4], const int64_t k_strides[4],
+                             float scale, int cls_n, void *hip_stream);
+
+/* Causal column means for one sequence (batch 1), fp16 inputs, fp32 output.
+ *   q          (1,H,Q_len,D), k (1,H,K_len,D) fp16; strides as above (index 0 ignored).
+ *   out        (K_len) fp32; receives the means over the H*Q_len rows.
+ *   k_past     number of keys every query may see before its own position: key j is
+ *              visible to query i  <=>  j <= k_past + i.  The reference infers
+ *              max(0, K_len - Q_len); pass that for drop-in behaviour.
+ * Replaces `_flash_colsum_causal(Q, K, scale, K_past)` including its host epilogue
+ * (reference: flash_colsum/kernel_causal.py:94-125; called from flash_colsum/ops.py:89). */
+int fcs_colsum_causal_f16(const void *q, const void *k, float *out, void *ws, size_t ws_bytes,
+                          int H, int Q_len, int K_len, int D, int k_past,
+                          const int64_t q_strides[4], const int64_t k_strides[4],
+                          float scale, void *hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASH_COLSUM_H */
