@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention column-mean hot path on one MI355X.
+
+A step is one call of `flash_colsum(Q, K, ...)` on synthetic inputs that are already
+resident in HBM.  The default workload is the batched non-causal self-attention shape
+B=8, H=16, S=2048, D=64 with K = Q.clone().  Prints ONE JSON line on stdout; everything
+else goes to stderr.
+
+  value          effective TFLOP/s of the whole call (wall clock, launch + epilogue
+                 included), counting two QK^T passes: 4*B*H*Sq*Sk*D / t
+  ms_per_step    wall-clock milliseconds per call
+  roofline       kernels-only time of one call (HIP events on the launch stream around the
+                 C-ABI call with output and workspace preallocated) against the dense
+                 fp16 MFMA peak
+  cpu_baseline   the eager materialising baseline (oracle/naive_colsum.py, a port of the
+                 reference's naive path) on this host's cores, same workload
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "flash-colsum_amd"))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2516.6  # MI355X dense fp16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (q shape, k shape, kwargs, K = Q.clone())
+    "noncausal_b2_h4_s512_d64": ((2, 4, 512, 64), (2, 4, 512, 64), dict(scale=0.125), False),
+    "noncausal_b8_h16_s2048_d64": ((8, 16, 2048, 64), (8, 16, 2048, 64), dict(), True),
+    "cls1_b32_h16_s577_d64": ((32, 16, 577, 64), (32, 16, 577, 64), dict(cls_len=1), False),
+    "causal_h32_q128_k4096_d128": ((1, 32, 128, 128), (1, 32, 4096, 128), dict(is_causal=True), False),
+    "causal_h32_q128_k16384_d128": ((1, 32, 128, 128), (1, 32, 16384, 128), dict(is_causal=True), False),
+    "causal_h32_q512_k65536_d128_peaky": ((1, 32, 512, 128), (1, 32, 65536, 128), dict(is_causal=True), False),
+}
+DEFAULT = "noncausal_b8_h16_s2048_d64"
+
+
+def make_inputs(name):
+    """fp32 CPU tensors from a CPU generator (seed 0, Q drawn first), identical on every host."""
+    import torch
+
+    qs, ks, kwargs, same = WORKLOADS[name]
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(qs, generator=g, dtype=torch.float32)
+    if same:
+        k = q.clone()
+    else:
+        k = torch.randn(ks, generator=g, dtype=torch.float32)
+    if name.endswith("peaky"):
+        # four head-dim channels scaled x8; first 64 keys pushed +3 sigma along Q's mean direction
+        k[..., [7, 31, 64, 101]] *= 8.0
+        u = q[0].mean(dim=1)
+        u = u / u.norm(dim=-1, keepdim=True)
+        k[0, :, :64, :] += 3.0 * u[:, None, :]
+    return q, k, kwargs
+
+
+def flops(name):
+    qs, ks, _, _ = WORKLOADS[name]
+    b, h, sq, d = qs
+    return 4.0 * b * h * sq * ks[2] * d
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=25)
+    ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one MI355X: this path has no multi-GPU part, run with --gpus 1")
+
+    import torch
+    from flash_colsum import flash_colsum, _hip
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    name = args.workload
+    q32, k32, kwargs = make_inputs(name)
+    q = q32.half().cuda()
+    k = k32.half().cuda()
+    torch.cuda.synchronize()
+
+    # ---- whole-call wall clock (the headline): K calls back to back between two syncs
+    for _ in range(args.warmup):
+        flash_colsum(q, k, **kwargs)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        flash_colsum(q, k, **kwargs)
+    torch.cuda.synchronize()
+    ms_call = (time.perf_counter() - t0) * 1e3 / args.steps
+    fl = flops(name)
+    tflops = fl / (ms_call * 1e-3) / 1e12
+
+    # ---- kernels only: HIP events on the launch stream around the C-ABI call
+    b, h, sq, d = q.shape
+    sk = k.shape[2]
+    causal = bool(kwargs.get("is_causal", False))
+    cls_n = int(kwargs.get("cls_len") or -1)
+    scale = float(kwargs.get("scale") or d ** -0.5)
+    lib = _hip.lib()
+    n_ws = _hip.workspace_bytes(causal, b, h, sq, sk, d, cls_n)
+    ws = torch.empty(max(n_ws, 1), dtype=torch.uint8, device="cuda")
+    out = torch.empty((b, sk), dtype=torch.float32, device="cuda")
+    qs_, ks_ = _hip._I64x4(*q.stride()), _hip._I64x4(*k.stride())
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        if causal:
+            rc = lib.fcs_colsum_causal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), ws.data_ptr(), n_ws,
+                                           h, sq, sk, d, max(0, sk - sq), qs_, ks_, scale, stream)
+        else:
+            rc = lib.fcs_colsum_noncausal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), ws.data_ptr(), n_ws,
+                                              b, h, sq, d, qs_, ks_, scale, cls_n, stream)
+        if rc != 0:
+            raise RuntimeError(_hip.strerror(rc))
+
+    for _ in range(args.warmup):
+        launch()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for e0, e1 in evs:
+        e0.record()
+        launch()
+        e1.record()
+    torch.cuda.synchronize()
+    ker_ms = statistics.mean(e0.elapsed_time(e1) for e0, e1 in evs)
+    ker_tflops = fl / (ker_ms * 1e-3) / 1e12
+    roofline = {
+        "bound": "mfma",
+        "kernel": "all kernels of one call (fcs_rowstats + fcs_colsum + fcs_finalize)",
+        "achieved": round(ker_tflops, 2),
+        "peak": PEAK_FP16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(ker_tflops / PEAK_FP16_TFLOPS, 4),
+        "kernel_ms": round(ker_ms, 5),
+        "algorithmic_flops": fl,
+        "traffic": None,
+    }
+    print(f"[bench] {name}: {ms_call:.4f} ms/call wall, {ker_ms:.4f} ms kernels, "
+          f"{tflops:.1f} / {ker_tflops:.1f} TFLOP/s", file=sys.stderr)
+
+    # ---- CPU baseline: eager materialising path on the host cores, same workload
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import naive_colsum
+
+        qc, kc = q32.half().float(), k32.half().float()
+        naive_colsum(qc, kc, **kwargs)
+        ts = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            naive_colsum(qc, kc, **kwargs)
+            ts.append(time.perf_counter() - t0)
+        t_cpu = statistics.median(ts)
+        cpu = {
+            "value": round(fl / t_cpu / 1e12, 5),
+            "unit": "TFLOP/s",
+            "ms_per_call": round(t_cpu * 1e3, 2),
+            "cores": torch.get_num_threads(),
+            "host_cpus": os.cpu_count(),
+            "kind": "port",
+            "sample": f"full workload {name}, fp32 torch eager on CPU, 1 warm-up + median of 3 calls",
+        }
+        print(f"[bench] cpu baseline: {t_cpu * 1e3:.1f} ms/call on {torch.get_num_threads()} threads", file=sys.stderr)
+
+    rec = {
+        "metric": "effective TFLOP/s (4*B*H*Sq*Sk*D per call, two QK^T passes) and ms/call, B8 H16 S2048 D64 non-causal"
+        if name == DEFAULT else f"effective TFLOP/s and ms/call, {name}",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_call, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp16 MFMA inputs, fp32 accumulate/softmax",
+        "data": "synthetic: N(0,1) from torch.Generator(seed 0) on CPU, rounded to fp16",
+        "config": {"workload": name, "q_shape": list(q.shape), "k_shape": list(k.shape), **{k_: v for k_, v in kwargs.items()}},
+        "frac_of_fp16_mfma_peak": round(tflops / PEAK_FP16_TFLOPS, 4),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(rec), flush=True)
+
+
+if __name__ == "__main__":
+    main()

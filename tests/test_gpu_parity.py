@@ -1,0 +1,301 @@
+"""GPU parity: the HIP path against the CPU oracle on the same seeded inputs.
+
+Bar (stated by the task): on the kernels' fp32 means, max |diff| <= 1e-4 AND element-wise
+relative error <= 1e-3, against an fp32/fp64 reference fed the same fp16-rounded inputs.
+Shapes mirror the reference's own tests (reference: tests/test_core.py:21-134), the five
+benchmark configurations, and the shapes the reference kernels get wrong (S not a
+multiple of the tile, D = 128, Q_len not a multiple of 16, cls_len > S).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 1e-4, 1e-3
+
+
+def _inputs(qs, ks, seed=0, same=False):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(qs, generator=g, dtype=torch.float32).half()
+    k = q.clone() if same else torch.randn(ks, generator=g, dtype=torch.float32).half()
+    return q, k
+
+
+def _assert_close(out, ref, what=""):
+    out = out.detach().cpu().double()
+    ref = ref.detach().cpu().double()
+    assert out.shape == ref.shape, (what, out.shape, ref.shape)
+    assert torch.isfinite(out).all(), what
+    err = (out - ref).abs()
+    rel = err / ref.abs().clamp_min(1e-9)
+    assert err.max().item() <= ATOL, f"{what}: max abs {err.max().item():.3e}"
+    assert rel.max().item() <= RTOL, f"{what}: max rel {rel.max().item():.3e}"
+
+
+def _run(q, k, **kw):
+    from flash_colsum import flash_colsum_f32
+
+    out = flash_colsum_f32(q.cuda(), k.cuda(), **kw)
+    torch.cuda.synchronize()
+    return out
+
+
+def _oracle(q, k, **kw):
+    from oracle import colsum_exact
+
+    return colsum_exact(q, k, **kw)
+
+
+# ---------------------------------------------------------------------------------------
+# committed golden vectors, through the C ABI directly
+# ---------------------------------------------------------------------------------------
+def test_golden_vectors_through_c_abi(golden):
+    from flash_colsum import _hip
+
+    lib = _hip.lib()
+    for name, c in golden.items():
+        q = torch.from_numpy(c["q"]).cuda().contiguous()
+        k = torch.from_numpy(c["k"]).cuda().contiguous()
+        b, h, sq, d = q.shape
+        sk = k.shape[2]
+        scale = c["scale"] if c["scale"] is not None else d ** -0.5
+        cls_n = -1 if c["cls_len"] is None else c["cls_len"]
+        n_ws = lib.fcs_workspace_bytes(int(c["causal"]), b, h, sq, sk, d, cls_n)
+        ws = torch.empty(max(n_ws, 1), dtype=torch.uint8, device="cuda")
+        out = torch.full((b, sk), float("nan"), dtype=torch.float32, device="cuda")
+        qs, ks = (ctypes.c_int64 * 4)(*q.stride()), (ctypes.c_int64 * 4)(*k.stride())
+        stream = torch.cuda.current_stream().cuda_stream
+        if c["causal"]:
+            rc = lib.fcs_colsum_causal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), ws.data_ptr(), n_ws, h, sq, sk,
+                                           d, max(0, sk - sq), qs, ks, scale, stream)
+        else:
+            rc = lib.fcs_colsum_noncausal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), ws.data_ptr(), n_ws, b, h,
+                                              sq, d, qs, ks, scale, cls_n, stream)
+        assert rc == 0, (name, _hip.strerror(rc))
+        torch.cuda.synchronize()
+        _assert_close(out, torch.from_numpy(c["out"]), name)
+
+
+# ---------------------------------------------------------------------------------------
+# the five benchmark configurations
+# ---------------------------------------------------------------------------------------
+def test_cfg1_small_noncausal_fp32_oracle():
+    g = torch.Generator().manual_seed(0)
+    q32 = torch.randn((2, 4, 512, 64), generator=g)
+    k32 = torch.randn((2, 4, 512, 64), generator=g)
+    from oracle import naive_colsum
+
+    out = _run(q32.half(), k32.half(), scale=1 / 8)
+    _assert_close(out, naive_colsum(q32.half().float(), k32.half().float(), scale=1 / 8), "cfg1 vs fp32 naive")
+    _assert_close(out, _oracle(q32.half(), k32.half(), scale=1 / 8), "cfg1 vs float64")
+    assert out.shape == (2, 512)
+
+
+def test_cfg2_batched_self_attention():
+    q, k = _inputs((8, 16, 2048, 64), None, same=True)
+    out = _run(q, k)
+    assert out.shape == (8, 2048)
+    _assert_close(out, _oracle(q, k), "cfg2")
+
+
+def test_cfg3_cls_token():
+    q, k = _inputs((32, 16, 577, 64), (32, 16, 577, 64))
+    out = _run(q, k, cls_len=1)
+    assert out.shape == (32, 577)
+    _assert_close(out, _oracle(q, k, cls_len=1), "cfg3")
+
+
+@pytest.mark.parametrize("k_len", [4096, 16384])
+def test_cfg4_causal_decode_window(k_len):
+    q, k = _inputs((1, 32, 128, 128), (1, 32, k_len, 128))
+    out = _run(q, k, is_causal=True)
+    assert out.shape == (1, k_len)
+    _assert_close(out, _oracle(q, k, is_causal=True), f"cfg4 K_len={k_len}")
+
+
+def _peaky(q32, k32, bias):
+    k32 = k32.clone()
+    k32[..., [7, 31, 64, 101]] *= 8.0
+    u = q32[0].mean(dim=1)
+    u = u / u.norm(dim=-1, keepdim=True)
+    k32[0, :, :64, :] += bias * u[:, None, :]
+    return k32
+
+
+def test_cfg5_long_context_peaky():
+    g = torch.Generator().manual_seed(0)
+    q32 = torch.randn((1, 32, 512, 128), generator=g)
+    k32 = _peaky(q32, torch.randn((1, 32, 65536, 128), generator=g), 3.0)
+    q, k = q32.half(), k32.half()
+    out = _run(q, k, is_causal=True)
+    assert out.shape == (1, 65536)
+    _assert_close(out, _oracle(q, k, is_causal=True), "cfg5")
+
+
+def test_strong_attention_sinks():
+    """Sink keys far above the row mean (bias 40 along Q's mean direction): a handful of
+    columns take most of the mass, the rest are tiny."""
+    g = torch.Generator().manual_seed(1)
+    q32 = torch.randn((1, 8, 256, 128), generator=g) + 0.5
+    k32 = _peaky(q32, torch.randn((1, 8, 8192, 128), generator=g), 40.0)
+    q, k = q32.half(), k32.half()
+    out = _run(q, k, is_causal=True)
+    ref = _oracle(q, k, is_causal=True)
+    assert ref[0, :64].sum() > 0.5
+    _assert_close(out, ref, "sinks")
+
+
+# ---------------------------------------------------------------------------------------
+# the reference's own test shapes (tests/test_core.py)
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape,kw", [
+    ((4, 8, 512, 64), {}),
+    ((1, 16, 8192, 64), {}),
+    ((4, 8, 512, 64), {"cls_len": 1}),
+    ((1, 16, 4096, 64), {"cls_len": 2}),
+])
+def test_reference_noncausal_cases(shape, kw):
+    q, k = _inputs(shape, shape)
+    out = _run(q, k, **kw)
+    assert out.shape == (shape[0], shape[2])
+    _assert_close(out, _oracle(q, k, **kw), f"{shape} {kw}")
+
+
+def test_reference_causal_case():
+    q, k = _inputs((1, 16, 128, 128), (1, 16, 16384, 128))
+    out = _run(q, k, is_causal=True)
+    assert out.shape == (1, 16384)
+    _assert_close(out, _oracle(q, k, is_causal=True), "reference causal")
+
+
+def test_reference_error_handling():
+    from flash_colsum import flash_colsum
+
+    q = torch.randn(2, 8, 128, 64, device="cuda", dtype=torch.float16)
+    k = torch.randn(2, 8, 1024, 64, device="cuda", dtype=torch.float16)
+    with pytest.raises(ValueError, match="batch size 1"):
+        flash_colsum(q, k, is_causal=True)
+    with pytest.raises(ValueError, match="CUDA"):
+        flash_colsum(torch.randn(1, 8, 128, 64), torch.randn(1, 8, 128, 64))
+    k = torch.randn(2, 8, 256, 64, device="cuda", dtype=torch.float16)
+    with pytest.raises(ValueError, match="same shape"):
+        flash_colsum(q, k)
+    with pytest.raises(RuntimeError, match="head dim"):
+        flash_colsum(torch.randn(1, 2, 16, 48, device="cuda", dtype=torch.float16),
+                     torch.randn(1, 2, 16, 48, device="cuda", dtype=torch.float16))
+
+
+# ---------------------------------------------------------------------------------------
+# edges: ragged sizes, tails, alignment, degenerate rows
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("qs,ks,kw", [
+    ((1, 1, 1, 64), (1, 1, 1, 64), {}),
+    ((2, 3, 31, 64), (2, 3, 31, 64), {}),
+    ((2, 3, 33, 128), (2, 3, 33, 128), {}),
+    ((3, 4, 577, 64), (3, 4, 577, 64), {}),
+    ((3, 4, 577, 64), (3, 4, 577, 64), {"cls_len": 3}),
+    ((2, 2, 100, 64), (2, 2, 100, 64), {"cls_len": 1000}),
+    ((2, 2, 300, 64), (2, 2, 300, 64), {"cls_len": 129}),
+    ((2, 2, 257, 128), (2, 2, 257, 128), {"scale": 0.3}),
+    ((1, 4, 100, 128), (1, 4, 1000, 128), {"is_causal": True}),
+    ((1, 4, 1, 64), (1, 4, 777, 64), {"is_causal": True}),
+    ((1, 4, 200, 64), (1, 4, 200, 64), {"is_causal": True}),
+    ((1, 4, 200, 64), (1, 4, 50, 64), {"is_causal": True}),
+    ((1, 4, 65, 128), (1, 4, 64, 128), {"is_causal": True}),
+    ((1, 2, 300, 64), (1, 2, 5000, 64), {"is_causal": True}),
+    ((1, 3, 17, 64), (1, 3, 17, 64), {}),
+    ((2, 2, 64, 64), (2, 2, 64, 64), {"scale": -0.3}),
+    ((2, 2, 64, 64), (2, 2, 64, 64), {"scale": 0.0}),
+    ((1, 2, 90, 64), (1, 2, 400, 64), {"is_causal": True, "scale": 0.0}),
+    ((2, 2, 200, 64), (2, 2, 200, 64), {"scale": 40.0}),
+])
+def test_edge_shapes(qs, ks, kw):
+    q, k = _inputs(qs, ks, seed=3)
+    _assert_close(_run(q, k, **kw), _oracle(q, k, **kw), f"{qs} {ks} {kw}")
+
+
+def test_explicit_k_past():
+    """The causal launcher's K_past argument (reference: kernel_causal.py:94-113)."""
+    from flash_colsum import _hip
+
+    q, k = _inputs((1, 3, 40, 64), (1, 3, 200, 64), seed=4)
+    for k_past in (0, 37, 160, 199, 500):
+        out = _hip.colsum_causal_f32(q.cuda(), k.cuda(), 0.125, K_past=k_past)
+        s = (q.double() @ k.double().transpose(-1, -2)) * 0.125
+        i = torch.arange(40).view(-1, 1)
+        j = torch.arange(200).view(1, -1)
+        p = torch.softmax(s.masked_fill(j > i + k_past, float("-inf")), -1)
+        _assert_close(out, p.mean((1, 2)), f"k_past={k_past}")
+
+
+def test_strided_and_unaligned_inputs():
+    g = torch.Generator().manual_seed(5)
+    base_q = torch.randn((2, 150, 4, 64), generator=g).half().cuda()   # (B, S, H, D) storage
+    base_k = torch.randn((2, 150, 4, 64), generator=g).half().cuda()
+    q, k = base_q.permute(0, 2, 1, 3), base_k.permute(0, 2, 1, 3)       # no copy needed
+    ref = _oracle(q.cpu(), k.cpu())
+    _assert_close(_run(q, k), ref, "permuted")
+    wide = torch.zeros((2, 4, 150, 128), dtype=torch.float16, device="cuda")
+    wide[..., ::2] = q
+    _assert_close(_run(wide[..., ::2], k), ref, "strided last dim (copied by the host layer)")
+    pad = torch.zeros((2, 4, 150, 72), dtype=torch.float16, device="cuda")
+    pad[..., 4:68] = k
+    _assert_close(_run(q, pad[..., 4:68]), ref, "rows not 16-byte aligned (copied by the host layer)")
+    every_other = torch.randn((2, 4, 300, 64), generator=g).half().cuda()
+    _assert_close(_run(every_other[:, :, ::2], every_other[:, :, ::2]),
+                  _oracle(every_other[:, :, ::2].cpu(), every_other[:, :, ::2].cpu()), "row stride 2*D")
+
+
+def test_deterministic_bits():
+    q, k = _inputs((2, 8, 700, 64), (2, 8, 700, 64), seed=6)
+    a = _run(q, k)
+    for _ in range(3):
+        assert torch.equal(a, _run(q, k))
+    q, k = _inputs((1, 8, 128, 128), (1, 8, 6000, 128), seed=7)
+    a = _run(q, k, is_causal=True)
+    for _ in range(3):
+        assert torch.equal(a, _run(q, k, is_causal=True))
+
+
+def test_public_api_returns_fp16_like_the_reference():
+    from flash_colsum import flash_colsum, flash_colsum_f32
+
+    q, k = _inputs((4, 8, 512, 64), (4, 8, 512, 64))
+    out = flash_colsum(q.cuda(), k.cuda())
+    assert out.dtype == torch.float16 and out.shape == (4, 512) and out.is_cuda
+    assert torch.equal(out, flash_colsum_f32(q.cuda(), k.cuda()).half())
+    ref = _oracle(q, k)
+    assert torch.allclose(out.cpu().double(), ref, atol=1e-3, rtol=1e-3)   # the reference's own bar
+    q, k = _inputs((1, 16, 128, 128), (1, 16, 4096, 128))
+    out = flash_colsum(q.cuda(), k.cuda(), is_causal=True)
+    assert out.dtype == torch.float16 and out.shape == (1, 4096)
+    out = flash_colsum(q.cuda(), q.cuda(), cls_len=2)
+    assert out.shape == (1, 128)
+    # non-fp16 inputs are accepted (converted on the device)
+    out32 = flash_colsum_f32(q.float().cuda(), k.float().cuda(), is_causal=True)
+    _assert_close(out32, _oracle(q, k, is_causal=True), "fp32 inputs")
+
+
+# ---------------------------------------------------------------------------------------
+# size-independent properties at the full benchmark sizes
+# ---------------------------------------------------------------------------------------
+def test_full_size_properties():
+    q, k = _inputs((8, 16, 2048, 64), None, same=True)
+    qc, kc = q.cuda(), k.cuda()
+    out = _run(qc, kc)
+    assert torch.allclose(out.double().sum(-1), torch.ones(8, dtype=torch.float64, device="cuda"), atol=1e-5)
+    perm = torch.randperm(2048, generator=torch.Generator().manual_seed(1)).cuda()
+    out_p = _run(qc, kc[:, :, perm])
+    _assert_close(out_p, out[:, perm], "key permutation")
+    out_h = _run(qc[:, torch.arange(15, -1, -1)], kc[:, torch.arange(15, -1, -1)])
+    _assert_close(out_h, out, "head permutation")
+    g = torch.Generator().manual_seed(0)
+    q5 = torch.randn((1, 32, 512, 128), generator=g).half().cuda()
+    k5 = torch.randn((1, 32, 65536, 128), generator=g).half().cuda()
+    out5 = _run(q5, k5, is_causal=True)
+    assert abs(out5.double().sum().item() - 1.0) < 1e-5
+    # the last key is visible to the last query only: its column mean is at most 1/(Q_len)
+    assert 0 < out5[0, -1].item() <= 1.0 / 512

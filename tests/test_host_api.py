@@ -1,0 +1,116 @@
+"""CPU-side tests: the public operator's validation (reference: flash_colsum/ops.py:58-97,
+tests/test_core.py:113-134), the C-ABI library's exports and its host-side argument checks.
+No kernel is launched here."""
+import ctypes
+import os
+import re
+import types
+
+import pytest
+import torch
+
+import flash_colsum
+from flash_colsum import _hip, flash_colsum as op
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+class FakeCuda:
+    """Stands in for a GPU tensor in validation tests: only what the checks read."""
+
+    def __init__(self, *shape):
+        self.shape = torch.Size(shape)
+        self.ndim = len(shape)
+        self.device = types.SimpleNamespace(type="cuda")
+
+
+def test_exports_match_reference_package():
+    assert callable(flash_colsum.flash_colsum) and callable(flash_colsum.naive_colsum)
+    assert flash_colsum.__version__ == "1.0.0"
+
+
+def test_validation_messages_and_order():
+    with pytest.raises(ValueError, match="4D"):
+        op(torch.zeros(2, 3, 4), torch.zeros(2, 3, 4))
+    # device check comes before every shape check (ops.py:62)
+    with pytest.raises(ValueError, match="CUDA"):
+        op(torch.zeros(1, 8, 128, 64), torch.zeros(1, 8, 128, 64))
+    with pytest.raises(ValueError, match="CUDA"):
+        op(torch.zeros(2, 8, 128, 64), torch.zeros(2, 8, 256, 64), is_causal=True, cls_len=0)
+    # cls_len checks come before the causal batch check (ops.py:65-68)
+    with pytest.raises(ValueError, match="only supported for non-causal"):
+        op(FakeCuda(2, 8, 128, 64), FakeCuda(2, 8, 1024, 64), is_causal=True, cls_len=1)
+    with pytest.raises(ValueError, match="must be positive"):
+        op(FakeCuda(2, 8, 128, 64), FakeCuda(2, 8, 256, 64), cls_len=0)
+    with pytest.raises(ValueError, match="batch size 1"):
+        op(FakeCuda(2, 8, 128, 64), FakeCuda(2, 8, 1024, 64), is_causal=True)
+    with pytest.raises(ValueError, match="same heads and head_dim"):
+        op(FakeCuda(1, 8, 128, 64), FakeCuda(1, 4, 1024, 64), is_causal=True)
+    with pytest.raises(ValueError, match="same heads and head_dim"):
+        op(FakeCuda(1, 8, 128, 64), FakeCuda(1, 8, 1024, 128), is_causal=True)
+    with pytest.raises(ValueError, match="same shape"):
+        op(FakeCuda(2, 8, 128, 64), FakeCuda(2, 8, 256, 64))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "flash_colsum.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fcs_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _hip.lib()
+    names = _declared_symbols()
+    assert names == ["fcs_abi_version", "fcs_colsum_causal_f16", "fcs_colsum_noncausal_f16", "fcs_strerror",
+                     "fcs_workspace_bytes"]
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert lib.fcs_abi_version() == 1
+
+
+def test_strerror_is_total():
+    for code in range(-8, 3):
+        assert isinstance(_hip.strerror(code), str) and _hip.strerror(code)
+    assert "head dim" in _hip.strerror(-3)
+
+
+def test_workspace_bytes():
+    wb = _hip.workspace_bytes
+    assert wb(False, 0, 1, 1, 1, 64) == 0 and wb(False, 1, 1, 1, 0, 64) == 0
+    for args in [(False, 8, 16, 2048, 2048, 64, -1), (False, 32, 16, 577, 577, 64, 1),
+                 (True, 1, 32, 128, 4096, 128, -1), (True, 1, 32, 512, 65536, 128, -1), (False, 1, 1, 1, 1, 64, -1)]:
+        n = wb(*args)
+        assert n > 0 and n % 256 == 0
+    # never more than a few floats per (row, head) plus a few partial outputs: O(S), not O(S^2)
+    assert wb(False, 8, 16, 2048, 2048, 64) < 64 << 20
+    assert wb(True, 1, 32, 512, 65536, 128) < 64 << 20
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    lib = _hip.lib()
+    st = (ctypes.c_int64 * 4)(8 * 16 * 64, 16 * 64, 64, 1)
+    bad_last = (ctypes.c_int64 * 4)(8 * 16 * 64, 16 * 64, 64, 2)
+    unaligned = (ctypes.c_int64 * 4)(8 * 16 * 66, 16 * 66, 66, 1)
+    p = ctypes.c_void_p(4096)  # never dereferenced: every call below fails its host checks
+    nc, ca = lib.fcs_colsum_noncausal_f16, lib.fcs_colsum_causal_f16
+    assert nc(None, p, p, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
+    assert nc(p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
+    assert nc(p, p, p, p, 1 << 30, 0, 8, 16, 64, st, st, 0.125, -1, None) == -2
+    assert nc(p, p, p, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, 0, None) == -2
+    assert nc(p, p, p, p, 1 << 30, 2, 8, 16, 80, st, st, 0.125, -1, None) == -3
+    assert nc(p, p, p, p, 1 << 30, 2, 8, 16, 64, bad_last, st, 0.125, -1, None) == -4
+    assert nc(p, p, p, p, 1 << 30, 2, 8, 16, 64, st, unaligned, 0.125, -1, None) == -4
+    assert nc(ctypes.c_void_p(4098), p, p, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -4
+    assert nc(p, p, p, p, 16, 2, 8, 16, 64, st, st, 0.125, -1, None) == -5
+    assert nc(p, p, p, None, 0, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
+    assert nc(p, p, p, p, 1 << 30, 2, 8, 16, 64, st, st, float("nan"), -1, None) == -6
+    assert ca(p, p, p, p, 1 << 30, 8, 16, 64, 64, -1, st, st, 0.125, None) == -2
+    assert ca(p, p, p, p, 1 << 30, 8, 16, 64, 96, 48, st, st, 0.125, None) == -3
+    assert ca(p, p, p, p, 16, 8, 16, 64, 64, 48, st, st, 0.125, None) == -5
+
+
+def test_missing_library_is_loud(monkeypatch, tmp_path):
+    monkeypatch.setattr(_hip, "_lib", None)
+    monkeypatch.setattr(_hip, "_LIB_PATH", str(tmp_path / "libflashcolsum.so"))
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _hip.lib()
