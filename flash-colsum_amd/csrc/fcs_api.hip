@@ -54,6 +54,8 @@ int run(int causal, const void *q, const void *k, float *out, void *ws, size_t w
     a.partial = reinterpret_cast<float *>(w + p.off_partial);
     a.out = out;
     a.inv_norm = 1.0f / ((float)H * (float)p.q_rows);
+    a.n_partials = p.n_partials;
+    a.f_kg = p.f_kg; a.f_tpw = p.f_tpw; a.f_nqblk = p.f_nqblk; a.f_hpg = p.f_hpg;
     return fcs::launch_colsum(p, a, stream);
 }
 

@@ -1,0 +1,43 @@
+// Small device helpers shared by the kernel files.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fcs {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+static constexpr float kNegBig = -1.0e30f;  // "hidden" score: finite so that max/sub never make NaN
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+__device__ __forceinline__ half8 load8(const _Float16 *p) { return *reinterpret_cast<const half8 *>(p); }
+
+__device__ __forceinline__ half8 flip_sign(half8 v)
+{
+    uint4v u = __builtin_bit_cast(uint4v, v);
+    u ^= 0x80008000u;
+    return __builtin_bit_cast(half8, u);
+}
+
+// Row of a 32x32 MFMA result tile held by accumulator register i of a lane in half-wave g
+// (the column is lane % 32).
+__device__ __forceinline__ int acc_row(int i, int g) { return 8 * (i >> 2) + 4 * g + (i & 3); }
+
+// value of the lane `lane ^ mask` for mask in {1, 2} (any values), or {4, 8} when the
+// value is already uniform over groups of `mask` lanes; DPP, no LDS traffic
+template <int CTRL>
+__device__ __forceinline__ float dpp_get(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+static constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
+static constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
+static constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7 - i within groups of 8
+static constexpr int kDppMirror = 0x140;      // lane i <-> 15 - i within rows of 16
+
+}  // namespace fcs

@@ -1,0 +1,371 @@
+// Attention column means on gfx950 (MI355X): fused single-kernel path for non-causal
+// calls whose whole key range fits in one workgroup's registers (S_k <= 2048, D = 64).
+//
+// One workgroup = 8 waves.  The waves form a (query group) x (key group) grid; a wave
+// computes the 32 x (32 * tiles) block of scores  S = Q_tile * K_tile^T  for its 32 query
+// rows and its keys with v_mfma_f32_32x32x16_f16 and KEEPS it in registers (up to 8
+// accumulator tiles = 128 VGPRs), so the scores are computed once and exponentiated
+// once.  In this orientation a lane owns one key (column l % 32) and 16 query rows, so the
+// column sums  sum_i e_ij / L_i  are in-lane FMAs; only the row sums L_i cross lanes and
+// waves, once per (head, row block), through a transpose-reduce in LDS.
+//
+// Q and K never pass through staging registers: every wave streams its own operands
+// with global_load_lds_dwordx4 into a private LDS ring, several tiles ahead of use, and
+// reads each 16-byte piece back into the lane that fetched it (so no layout or bank
+// question arises).  The DMA loads are waited for by hand with s_waitcnt vmcnt(n).
+//
+// Per (head, row block):
+//   phase 1  for each tile: MFMA -> e = 2^(c*s) -> in-lane partial row sums
+//   reduce   row sums over the 32 lanes x key-group waves (LDS), w_i = 1 / L_i
+//   phase 3  col_acc[tile] += sum_r e[tile][r] * w[r]
+// The exponent is taken WITHOUT max subtraction while that is exact in fp32: every row
+// sum must land in [2^-80, 2^120).  If any row of the workgroup falls outside (or is not
+// finite) the block redoes that (head, row block) with the usual max-subtracted softmax.
+// A workgroup walks over its heads and writes one partial column-sum slab at the end;
+// slabs have a single writer each and are added in index order by fcs_finalize_kernel.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fcs_device.h"
+#include "fcs_kernels.h"
+
+namespace fcs {
+
+namespace {
+
+constexpr float kSumLo = 8.2718061e-25f;   // 2^-80
+constexpr float kSumHi = 1.3292280e+36f;   // 2^120
+
+// Sum (MAX = false) or max (MAX = true) of v[16] over the 32 lanes of each half-wave and
+// over the key-group waves of the same query group.  In: v[i] belongs to row
+// acc_row(i, g) of the wave's 32 rows.  Out: the reduced value of every row lands in
+// row_out[query_group * 32 + row]; `post` maps (row index within block, value) to what is
+// stored.  Two barriers.  red: 8192 floats, row_out: 256 floats.
+template <bool MAX, typename Post>
+__device__ __forceinline__ void reduce_rows(const float (&v)[16], float *red, float *row_out, int kg_n, int qg, int kg,
+                                            int n, int g, int tid, Post post)
+{
+    const int vals_per_row = kg_n * 32;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) red[(qg * 32 + acc_row(i, g)) * vals_per_row + kg * 32 + n] = v[i];
+    __syncthreads();
+    {
+        const int tpr = 2 * kg_n;  // threads per row: each folds 16 of the row's 32*kg_n values
+        const int row = tid / tpr, sub = tid - row * tpr;
+        const floatx4 *src = reinterpret_cast<const floatx4 *>(red + row * vals_per_row);
+        float s = MAX ? kNegBig : 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const floatx4 x = src[c * tpr + sub];
+            if (MAX)
+                s = fmaxf(fmaxf(fmaxf(s, x[0]), fmaxf(x[1], x[2])), x[3]);
+            else
+                s += (x[0] + x[1]) + (x[2] + x[3]);
+        }
+        // fold the tpr (2, 4, 8 or 16) neighbouring lanes; every lane ends with the total
+        float o = dpp_get<kDppXor1>(s);
+        s = MAX ? fmaxf(s, o) : s + o;
+        if (tpr >= 4) { o = dpp_get<kDppXor2>(s); s = MAX ? fmaxf(s, o) : s + o; }
+        if (tpr >= 8) { o = dpp_get<kDppHalfMirror>(s); s = MAX ? fmaxf(s, o) : s + o; }
+        if (tpr >= 16) { o = dpp_get<kDppMirror>(s); s = MAX ? fmaxf(s, o) : s + o; }
+        const float res = post(row, s);
+        if (sub == 0) row_out[row] = res;
+    }
+    __syncthreads();
+}
+
+}  // namespace
+
+#define FCS_GLDS16(gptr, lptr)                                                                   \
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gptr),    \
+                                     (__attribute__((address_space(3))) void *)(lptr), 16, 0, 0)
+#define FCS_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
+// stops the compiler from precomputing per-tile values of a scalar for the whole walk
+#define FCS_OPAQUE_S(x) asm volatile("" : "+s"(x))
+#define FCS_OPAQUE_V(x) asm volatile("" : "+v"(x))
+
+// RAGGED = false: S_k is exactly (key groups) x TPW x 32, no padding keys anywhere.
+// RAGGED = true : the last tiles may hold padding keys; every exponent is masked per lane.
+template <int D, int TPW, bool RAGGED>
+__global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
+{
+    static_assert(D == 64, "the fused path is laid out for 64-wide heads");
+    constexpr int NT = D / 16;             // MFMA steps (and 16-byte pieces per lane) per operand tile
+    constexpr int NS = 3;                  // ring slots per wave
+    constexpr int AHEAD = NS - 1;          // items in flight ahead of the one being consumed
+    constexpr int ITEMS = TPW + 1;         // per (head, row block): the Q tile, then TPW key tiles
+    constexpr int SLOT_BYTES = NT * 1024;  // one item: NT pieces x 64 lanes x 16 bytes
+    __shared__ __attribute__((aligned(16))) float red[8192];
+    __shared__ __attribute__((aligned(16))) float rowv[256];
+    __shared__ __attribute__((aligned(16))) char ring[8 * NS * SLOT_BYTES];
+    __shared__ int redo[2];
+
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what derives from it stays in SGPRs
+    const int kg_n = a.f_kg, qg_n = 8 / kg_n;
+    const int qg = wave / kg_n, kg = wave - qg * kg_n;
+    const int b = blockIdx.x % a.B, qblk = blockIdx.x / a.B;
+    const int hgi = blockIdx.y;
+    const int h_begin = hgi * a.f_hpg, h_end = min(a.H, h_begin + a.f_hpg);
+    const int n_units = h_end - h_begin;
+    const int blk_row0 = qblk * 32 * qg_n;  // first query row of the block
+    const int q0 = blk_row0 + qg * 32;      // first query row of this wave
+    const int kbase = kg * TPW * 32;        // first key of this wave
+    const int k_full = max(0, min(TPW, (a.Sk - kbase) / 32));  // key tiles of this wave without padding keys
+    const bool q_full = (q0 + 32 <= a.Sq);
+
+    if (tid < 2) redo[tid] = 0;
+    __syncthreads();
+
+    // Operand tiles are 32 rows x 64 halves (128 B per row).  One DMA instruction moves 8
+    // whole rows (1 KB, 8 full cache lines): lane L brings 16-byte piece L % 8 of row L / 8,
+    // and the 64 pieces land in the ring in lane order, i.e. the tile sits row-major in
+    // LDS.  To keep the later operand reads (32 lanes, 128 B apart) off each other's banks
+    // the pieces of a row are stored XOR-swizzled: position p of row r holds piece
+    // p ^ ((r >> 1) & 7).  The swizzle only depends on the parity of the instruction index.
+    int lrow = lane >> 3;  // row within the 8 rows of one DMA instruction
+    uint32_t piece_b[2];         // byte offset in its row of the piece this lane fetches (even / odd instruction)
+#pragma unroll
+    for (int par = 0; par < 2; ++par) piece_b[par] = (uint32_t)(((lane & 7) ^ ((par * 4 + (lane >> 4)) & 7)) * 16);
+    const uint32_t q_row_b = (uint32_t)a.qs_s * 2u, k_row_b = (uint32_t)a.ks_s * 2u;  // row pitch in bytes
+    uint32_t q_voff[2] = {lrow * q_row_b + piece_b[0], lrow * q_row_b + piece_b[1]};
+    uint32_t k_voff[2] = {lrow * k_row_b + piece_b[0], lrow * k_row_b + piece_b[1]};
+    const char *q_b = reinterpret_cast<const char *>(a.q + (int64_t)b * a.qs_b) + (int64_t)q0 * q_row_b;
+    const char *k_b = reinterpret_cast<const char *>(a.k + (int64_t)b * a.ks_b) + (int64_t)kbase * k_row_b;
+    const int64_t q_head_b = a.qs_h * 2, k_head_b = a.ks_h * 2;
+    char *my_ring = ring + wave * (NS * SLOT_BYTES);
+
+    // DMA rows [0, 32) of the tile starting at `tile` (uniform) into ring slot `slot`.
+    // `rows_left` <= 31 marks a tile that runs past the end of its tensor slice: such rows are
+    // replaced by the last real row (they are masked or ignored by the consumer).
+    auto fetch_tile = [&](const char *tile, uint32_t row_b, const uint32_t (&voff)[2], bool full, int rows_left, int slot) {
+        char *dst = my_ring + slot * SLOT_BYTES;
+        if (full) {
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) FCS_GLDS16(tile + (uint32_t)(tt * 8) * row_b + voff[tt & 1], dst + tt * 1024);
+        } else {
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) {
+                const int row = max(0, min(tt * 8 + lrow, rows_left - 1));
+                FCS_GLDS16(tile + (uint32_t)row * row_b + piece_b[tt & 1], dst + tt * 1024);
+            }
+        }
+    };
+    // read a ring slot back as an MFMA operand: lane (n, g) takes, for step tt, piece 2*tt + g of
+    // row n.  Issued from inline assembly: the compiler would otherwise make every LDS read wait
+    // for ALL outstanding DMA fetches (vmcnt(0)), which would undo the look-ahead.
+    uint32_t take_addr[NT];
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt)
+        take_addr[tt] = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)my_ring +
+                        (uint32_t)(n * 128 + (((2 * tt + g) ^ ((n >> 1) & 7)) * 16));
+    auto take = [&](int slot, half8 (&dst)[NT]) {
+        const uint32_t off = (uint32_t)(slot * SLOT_BYTES);
+        static_assert(NT == 4, "four pieces per lane");
+        asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&v"(dst[0]), "=&v"(dst[1]), "=&v"(dst[2]), "=&v"(dst[3])
+                     : "v"(take_addr[0] + off), "v"(take_addr[1] + off), "v"(take_addr[2] + off), "v"(take_addr[3] + off)
+                     : "memory");
+    };
+
+    float col_acc[TPW];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) col_acc[t] = 0.f;
+
+    // The walk: for every head the Q tile, then the TPW key tiles ("items").  Item i lives in
+    // ring slot i % NS; while item i is consumed, item i + AHEAD is fetched into the slot that
+    // item i - 1 just left.  Past the last head the fetches repeat it, so that the number of
+    // outstanding DMA instructions at every wait is a compile-time constant.
+    auto fetch_item = [&](const char *qh, const char *kh, int j, int slot) {  // j: position in the head, compile-time
+        if (j == 0)
+            fetch_tile(qh, q_row_b, q_voff, q_full, a.Sq - q0, slot);
+        else
+            fetch_tile(kh + (int64_t)((j - 1) * 32) * k_row_b, k_row_b, k_voff, (j - 1) < k_full, a.Sk - kbase - (j - 1) * 32, slot);
+    };
+
+    int cs = 0;  // slot of the item being consumed
+    {
+        const char *qh = q_b + (int64_t)h_begin * q_head_b, *kh = k_b + (int64_t)h_begin * k_head_b;
+        const char *qh1 = q_b + (int64_t)min(h_begin + 1, h_end - 1) * q_head_b, *kh1 = k_b + (int64_t)min(h_begin + 1, h_end - 1) * k_head_b;
+#pragma unroll
+        for (int i = 0; i < AHEAD; ++i) fetch_item(i < ITEMS ? qh : qh1, i < ITEMS ? kh : kh1, i % ITEMS, i % NS);
+    }
+
+    for (int unit = 0; unit < n_units; ++unit) {
+        // pointers of this head and of the next one (the last head repeats); kept opaque so that
+        // per-tile addresses are formed when needed instead of being held in registers
+        const int h = h_begin + unit, h1 = min(h + 1, h_end - 1);
+        const char *qh = q_b + (int64_t)h * q_head_b, *kh = k_b + (int64_t)h * k_head_b;
+        const char *qh1 = q_b + (int64_t)h1 * q_head_b, *kh1 = k_b + (int64_t)h1 * k_head_b;
+        uint32_t k_row_b_o = k_row_b;
+        FCS_OPAQUE_S(k_row_b_o);
+        (void)k_row_b_o;
+        FCS_OPAQUE_V(q_voff[0]); FCS_OPAQUE_V(q_voff[1]); FCS_OPAQUE_V(k_voff[0]); FCS_OPAQUE_V(k_voff[1]);
+        FCS_OPAQUE_V(piece_b[0]); FCS_OPAQUE_V(piece_b[1]); FCS_OPAQUE_V(lrow);
+
+        floatx16 acc[TPW];
+        float rs[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) rs[i] = 0.f;
+
+        // e = 2^(c*s) for tile t, in place, and its contribution to the row sums
+        auto exp_tile = [&](int t) {
+            if (!RAGGED) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float e = fast_exp2(acc[t][i] * a.c);
+                    acc[t][i] = e;
+                    rs[i] += e;
+                }
+            } else {
+                const bool real = (kbase + t * 32 + n) < a.Sk;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float e = real ? fast_exp2(acc[t][i] * a.c) : 0.f;
+                    acc[t][i] = e;
+                    rs[i] += e;
+                }
+            }
+        };
+        // one step of the walk: start the look-ahead fetch, wait for this item, read it back
+        auto step = [&](int j, half8 (&dst)[NT]) {
+            const int fj = (j + AHEAD) % ITEMS;
+            const bool next_head = (j + AHEAD) >= ITEMS;
+            const int fs = (cs == 0) ? NS - 1 : cs - 1;  // the slot item (this - 1) just left
+            fetch_item(next_head ? qh1 : qh, next_head ? kh1 : kh, fj, fs);
+            FCS_WAIT_VM(AHEAD * NT);
+            take(cs, dst);
+            cs = (cs == NS - 1) ? 0 : cs + 1;
+        };
+
+        // ---------------- phase 1
+        half8 qf[NT];
+        step(0, qf);
+        if (a.negate) {
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) qf[tt] = flip_sign(qf[tt]);
+        }
+#pragma unroll
+        for (int t = 0; t < TPW; ++t) {
+            half8 kf[NT];
+            step(1 + t, kf);
+            floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[tt], kf[tt], c, 0, 0, 0);
+            acc[t] = c;
+            if (t > 0) exp_tile(t - 1);  // VALU work of the previous tile runs under this tile's MFMAs
+        }
+        exp_tile(TPW - 1);
+
+        // ---------------- row sums over lanes and key-group waves; w = 1/L (0 for rows not averaged)
+        int *flag = &redo[unit & 1];
+        reduce_rows<false>(rs, red, rowv, kg_n, qg, kg, n, g, tid, [&](int row, float L) {
+            if (!(L >= kSumLo && L < kSumHi)) *flag = 1;
+            return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
+        });
+        const bool slow = (*flag != 0);
+        if (tid == 0) redo[(unit + 1) & 1] = 0;
+
+        if (slow) {
+            // ------------ rare: max-subtracted softmax for this (head, row block).  Operands are
+            // fetched again with ordinary loads (the ring keeps streaming ahead untouched).
+            const _Float16 *qp = reinterpret_cast<const _Float16 *>(qh) + (int64_t)min(n, a.Sq - 1 - q0) * a.qs_s + g * 8;
+            const _Float16 *kp = reinterpret_cast<const _Float16 *>(kh) + g * 8;
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) {
+                const half8 v = load8(qp + tt * 16);
+                qf[tt] = a.negate ? flip_sign(v) : v;
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) rs[i] = kNegBig;
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) {
+                half8 kf[NT];
+                const int krow = max(0, min(t * 32 + n, a.Sk - 1 - kbase));
+#pragma unroll
+                for (int tt = 0; tt < NT; ++tt) kf[tt] = load8(kp + (int64_t)krow * a.ks_s + tt * 16);
+                floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int tt = 0; tt < NT; ++tt) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[tt], kf[tt], c, 0, 0, 0);
+                acc[t] = c;
+                const bool real = (kbase + t * 32 + n) < a.Sk;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) rs[i] = fmaxf(rs[i], real ? c[i] : kNegBig);
+            }
+            reduce_rows<true>(rs, red, rowv, kg_n, qg, kg, n, g, tid, [&](int, float m) { return m; });
+#pragma unroll
+            for (int i = 0; i < 16; ++i) rs[i] = 0.f;
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const floatx4 m4 = *reinterpret_cast<const floatx4 *>(&rowv[qg * 32 + 8 * i4 + 4 * g]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float nm = -m4[j] * a.c;
+#pragma unroll
+                    for (int t = 0; t < TPW; ++t) {
+                        const bool real = (kbase + t * 32 + n) < a.Sk;
+                        const float e = real ? fast_exp2(fmaf(acc[t][4 * i4 + j], a.c, nm)) : 0.f;
+                        acc[t][4 * i4 + j] = e;
+                        rs[4 * i4 + j] += e;
+                    }
+                }
+            }
+            reduce_rows<false>(rs, red, rowv, kg_n, qg, kg, n, g, tid, [&](int row, float L) {
+                return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
+            });
+        }
+
+        // ---------------- phase 3: column sums of e * w
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+            const floatx4 w4 = *reinterpret_cast<const floatx4 *>(&rowv[qg * 32 + 8 * i4 + 4 * g]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int t = 0; t < TPW; ++t) col_acc[t] = fmaf(acc[t][4 * i4 + j], w4[j], col_acc[t]);
+            }
+        }
+    }
+    FCS_WAIT_VM(0);  // drain the look-ahead fetches before the block's LDS is released
+
+    // ---------------- the two half-waves hold different rows of the same keys: add, then store
+    const int slab = (hgi * a.f_nqblk + qblk) * qg_n + qg;
+    float *dst = a.partial + ((int64_t)slab * a.B + b) * a.Sk;
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+        const float v = col_acc[t] + __shfl_xor(col_acc[t], 32);
+        const int key = kbase + t * 32 + n;
+        if (g == 0 && key < a.Sk) dst[key] = v;
+    }
+}
+
+template <int TPW>
+static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
+{
+    const dim3 grid(p.f_nqblk * p.B, p.f_hg);
+    if (p.Sk == p.f_kg * TPW * 32)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false>), grid, dim3(512), 0, st, a);
+    else
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true>), grid, dim3(512), 0, st, a);
+}
+
+hipError_t launch_fused(const Plan &p, const Args &a, hipStream_t st)
+{
+    switch (p.f_tpw) {
+    case 1: launch_tpw<1>(p, a, st); break;
+    case 2: launch_tpw<2>(p, a, st); break;
+    case 3: launch_tpw<3>(p, a, st); break;
+    case 4: launch_tpw<4>(p, a, st); break;
+    case 5: launch_tpw<5>(p, a, st); break;
+    case 6: launch_tpw<6>(p, a, st); break;
+    case 7: launch_tpw<7>(p, a, st); break;
+    case 8: launch_tpw<8>(p, a, st); break;
+    default: return hipErrorInvalidValue;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return launch_finalize(a, st);
+}
+
+}  // namespace fcs

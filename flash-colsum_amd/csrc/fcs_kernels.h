@@ -26,9 +26,21 @@ struct Args {
     float *partial;  // [gh*gq][B][Sk]
     float *out;      // [B][Sk]
     float inv_norm;  // 1 / (H * q_rows)
+    int n_partials;  // slabs of `partial` that fcs_finalize_kernel adds up
+    // fused single-kernel path (scores stay in registers)
+    int f_kg;        // waves along the key axis (1, 2, 4 or 8); 8 / f_kg waves along the query axis
+    int f_tpw;       // 32-key tiles per wave (<= 8)
+    int f_nqblk;     // blocks along the query axis (32 * 8 / f_kg rows each)
+    int f_hpg;       // heads per block
 };
 
 // Enqueues every kernel of one call on `stream`; returns 0 or the hipError_t of a failed launch.
 int launch_colsum(const Plan &p, const Args &a, void *stream);
+
+// fused path, defined in fcs_fused.hip
+hipError_t launch_fused(const Plan &p, const Args &a, hipStream_t st);
+
+// shared final reduction out = inv_norm * sum of the n_partials slabs (fcs_kernels.hip)
+hipError_t launch_finalize(const Args &a, hipStream_t st);
 
 }  // namespace fcs

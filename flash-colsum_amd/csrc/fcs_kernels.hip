@@ -19,30 +19,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fcs_device.h"
 #include "fcs_kernels.h"
 
 namespace fcs {
-
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
-
-static constexpr float kNegBig = -1.0e30f;  // "hidden" score: finite so that max/sub never make NaN
-
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
-
-__device__ __forceinline__ half8 load8(const _Float16 *p) { return *reinterpret_cast<const half8 *>(p); }
-
-__device__ __forceinline__ half8 flip_sign(half8 v)
-{
-    uint4v u = __builtin_bit_cast(uint4v, v);
-    u ^= 0x80008000u;
-    return __builtin_bit_cast(half8, u);
-}
-
-// key (A-operand row) held by accumulator register i of a lane in half-wave g
-__device__ __forceinline__ int acc_row(int i, int g) { return 8 * (i >> 2) + 4 * g + (i & 3); }
 
 // ------------------------------------------------------------------------------------
 // pass 1: per-row log-sum-exp (or per-split partials)
@@ -362,7 +342,7 @@ __global__ __launch_bounds__(256) void fcs_finalize_kernel(const Args a)
     const int64_t n = (int64_t)a.B * a.Sk;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= n) return;
-    const int ng = a.gh * a.gq;
+    const int ng = a.n_partials;
     float s = 0.f;
     for (int gi = 0; gi < ng; ++gi) s += a.partial[(int64_t)gi * n + idx];
     a.out[idx] = s * a.inv_norm;
@@ -371,6 +351,13 @@ __global__ __launch_bounds__(256) void fcs_finalize_kernel(const Args a)
 // ------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------
+hipError_t launch_finalize(const Args &a, hipStream_t st)
+{
+    const int64_t n = (int64_t)a.B * a.Sk;
+    hipLaunchKernelGGL(fcs_finalize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
 template <int D>
 static hipError_t launch_d(const Plan &p, const Args &a, hipStream_t st)
 {
@@ -400,10 +387,7 @@ static hipError_t launch_d(const Plan &p, const Args &a, hipStream_t st)
         if (e != hipSuccess) return e;
     }
     if (p.gh * p.gq > 1) {
-        const int64_t n = (int64_t)p.B * p.Sk;
-        const dim3 grid((unsigned)((n + 255) / 256));
-        hipLaunchKernelGGL(fcs_finalize_kernel, grid, blk, 0, st, a);
-        hipError_t e = hipGetLastError();
+        hipError_t e = launch_finalize(a, st);
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -412,6 +396,7 @@ static hipError_t launch_d(const Plan &p, const Args &a, hipStream_t st)
 int launch_colsum(const Plan &p, const Args &a, void *stream)
 {
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (p.fused) return (int)launch_fused(p, a, st);
     hipError_t e = (p.D == 64) ? launch_d<64>(p, a, st) : launch_d<128>(p, a, st);
     return (int)e;
 }

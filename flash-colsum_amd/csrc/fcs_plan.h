@@ -10,6 +10,7 @@ namespace fcs {
 constexpr int kWavesPerBlock = 4;   // 256 threads
 constexpr int kStageKeys = 64;      // keys staged in LDS per step of the row-statistics pass
 constexpr int kStageRows = 64;      // query rows staged in LDS per step of the column pass
+constexpr int kFusedMaxKeys = 2048; // 8 waves x 8 tiles x 32 keys of fp32 scores per 32 query rows
 constexpr int kTargetBlocks = 1024; // 256 CUs x 4: enough workgroups to fill the chip twice over
 
 struct Plan {
@@ -27,6 +28,14 @@ struct Plan {
     int n_kblk;
     int gh, gq;      // groups along heads / along staged query tiles
     int heads_per_group, qtiles_per_group;
+    // fused single-kernel path: non-causal, all keys of a row block fit in one
+    // workgroup's registers.  grid = (f_nqblk * B, f_hg)
+    int fused;       // 1: use it (then the two-pass fields above are unused)
+    int f_kg, f_qg;  // waves along keys / along queries, f_kg * f_qg == 8
+    int f_tpw;       // 32-key tiles per wave
+    int f_nqblk;     // query blocks of 32 * f_qg rows
+    int f_hg, f_hpg; // head groups, heads per group
+    int n_partials;  // slabs summed by the finalize kernel
     // workspace layout (byte offsets, each 256-byte aligned)
     size_t off_lse;      // float  [B*H][rows_pad]            log2-domain log-sum-exp
     size_t off_ml;       // float2 [B*H][n_chunks][rows_pad]  only when n_chunks > 1
@@ -75,6 +84,30 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     if (gq < 1) gq = 1;
     p.qtiles_per_group = ceil_div(n_qt, gq);
     p.gq = ceil_div(n_qt, p.qtiles_per_group);
+
+    // ---- fused path
+    p.fused = 0;
+    p.n_partials = p.gh * p.gq;
+    if (!causal && Sk <= kFusedMaxKeys && D == 64) {
+        p.fused = 1;
+        const int tiles = ceil_div(Sk, 32);
+        p.f_kg = 1;
+        while (p.f_kg * 8 < tiles) p.f_kg *= 2;  // <= 8 tiles per wave
+        p.f_qg = 8 / p.f_kg;
+        p.f_tpw = ceil_div(tiles, p.f_kg);
+        p.f_nqblk = ceil_div(p.q_rows, 32 * p.f_qg);
+        const long basef = (long)p.f_nqblk * B;
+        int hg = (int)((512 + basef - 1) / basef);
+        if (hg > H) hg = H;
+        if (hg < 1) hg = 1;
+        p.f_hpg = ceil_div(H, hg);
+        p.f_hg = ceil_div(H, p.f_hpg);
+        p.n_partials = p.f_hg * p.f_nqblk * p.f_qg;
+        size_t off = align256(sizeof(float) * (size_t)p.n_partials * B * Sk);
+        p.off_lse = p.off_ml = p.off_partial = 0;
+        p.total = off;
+        return true;
+    }
 
     // ---- workspace
     size_t off = 0;
