@@ -7,16 +7,17 @@
 // accumulator tiles = 128 VGPRs), so the scores are computed once and exponentiated
 // once.  In this orientation a lane owns one key (column l % 32) and 16 query rows, so the
 // column sums  sum_i e_ij / L_i  are in-lane FMAs; only the row sums L_i cross lanes and
-// waves, once per (head, row block), through a transpose-reduce in LDS.
+// waves, once per (head, row block): lanes are folded by a wave-private transpose through
+// LDS, the key-group waves by one workgroup barrier.
 //
 // Q and K never pass through staging registers: every wave streams its own operands
 // with global_load_lds_dwordx4 into a private LDS ring, several tiles ahead of use, and
-// reads each 16-byte piece back into the lane that fetched it (so no layout or bank
-// question arises).  The DMA loads are waited for by hand with s_waitcnt vmcnt(n).
+// reads them back as MFMA operands.  The DMA loads are waited for by hand with
+// s_waitcnt vmcnt(n).
 //
 // Per (head, row block):
 //   phase 1  for each tile: MFMA -> e = 2^(c*s) -> in-lane partial row sums
-//   reduce   row sums over the 32 lanes x key-group waves (LDS), w_i = 1 / L_i
+//   reduce   row sums over the 32 lanes x key-group waves, w_i = 1 / L_i
 //   phase 3  col_acc[tile] += sum_r e[tile][r] * w[r]
 // The exponent is taken WITHOUT max subtraction while that is exact in fp32: every row
 // sum must land in [2^-80, 2^120).  If any row of the workgroup falls outside (or is not
@@ -33,56 +34,104 @@ namespace fcs {
 
 namespace {
 
-constexpr float kSumLo = 8.2718061e-25f;   // 2^-80
-constexpr float kSumHi = 1.3292280e+36f;   // 2^120
+constexpr float kSumLo = 8.2718061e-25f;  // 2^-80
+constexpr float kSumHi = 1.3292280e+36f;  // 2^120
+constexpr int kRedPitch = 40;             // floats per row of the wave-private transpose buffer
 
-// Sum (MAX = false) or max (MAX = true) of v[16] over the 32 lanes of each half-wave and
-// over the key-group waves of the same query group.  In: v[i] belongs to row
-// acc_row(i, g) of the wave's 32 rows.  Out: the reduced value of every row lands in
-// row_out[query_group * 32 + row]; `post` maps (row index within block, value) to what is
-// stored.  Two barriers.  red: 8192 floats, row_out: 256 floats.
+#define FCS_GLDS16(gptr, lptr)                                                                \
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gptr), \
+                                     (__attribute__((address_space(3))) void *)(lptr), 16, 0, 0)
+#define FCS_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
+// Hides a value's origin from the optimiser.  Used inside the walk over heads so that
+// per-tile addresses are formed where they are used instead of being precomputed for the
+// whole walk and held in (or spilled from) dozens of registers.
+#define FCS_OPAQUE_V(x) asm volatile("" : "+v"(x))
+
+// LDS scratch of one workgroup for the row reductions
+struct RowRed {
+    float *red_w;  // wave-private [32][kRedPitch]
+    float *part;   // [2][256]: per-wave row partials, double-buffered by reduction parity
+    float *wv_w;   // wave-private [32]: the reduced (and post-processed) value of each row
+    int parity;
+};
+
+// Reduces v[16] (v[i] belongs to row acc_row(i, g) of the wave's 32 rows) over the 32 lanes of
+// each half-wave and over the key-group waves of the same query group: sum, or max if MAX.
+// `post(row_in_block, total)` maps the total to what is left in rr.wv_w[row] for the lanes to
+// read back.  Returns (sum only) whether any row total of the WORKGROUP is outside
+// [2^-80, 2^120) or not finite; the answer is the same in every wave.  One barrier.
 template <bool MAX, typename Post>
-__device__ __forceinline__ void reduce_rows(const float (&v)[16], float *red, float *row_out, int kg_n, int qg, int kg,
-                                            int n, int g, int tid, Post post)
+__device__ __forceinline__ bool reduce_rows(const float (&v)[16], RowRed &rr, int kg_n, int qg, int kg, int lane, Post post)
 {
-    const int vals_per_row = kg_n * 32;
+    const int n = lane & 31, g = lane >> 5;
+    // lanes: transpose through the wave's own LDS block (LDS executes a wave's accesses in order)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) red[(qg * 32 + acc_row(i, g)) * vals_per_row + kg * 32 + n] = v[i];
-    __syncthreads();
+    for (int i = 0; i < 16; ++i) rr.red_w[acc_row(i, g) * kRedPitch + n] = v[i];
+    __builtin_amdgcn_wave_barrier();
+    const int row = lane >> 1, half = lane & 1;
+    float s;
     {
-        const int tpr = 2 * kg_n;  // threads per row: each folds 16 of the row's 32*kg_n values
-        const int row = tid / tpr, sub = tid - row * tpr;
-        const floatx4 *src = reinterpret_cast<const floatx4 *>(red + row * vals_per_row);
-        float s = MAX ? kNegBig : 0.f;
+        const floatx4 *src = reinterpret_cast<const floatx4 *>(rr.red_w + row * kRedPitch);
+        floatx4 x[4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const floatx4 x = src[c * tpr + sub];
-            if (MAX)
-                s = fmaxf(fmaxf(fmaxf(s, x[0]), fmaxf(x[1], x[2])), x[3]);
-            else
-                s += (x[0] + x[1]) + (x[2] + x[3]);
+        for (int c = 0; c < 4; ++c) x[c] = src[2 * c + half];
+        if (MAX) {
+            s = x[0][0];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) s = fmaxf(fmaxf(fmaxf(s, x[c][0]), fmaxf(x[c][1], x[c][2])), x[c][3]);
+            s = fmaxf(s, dpp_get<kDppXor1>(s));
+        } else {
+            s = ((x[0][0] + x[0][1]) + (x[0][2] + x[0][3])) + ((x[1][0] + x[1][1]) + (x[1][2] + x[1][3]));
+            s += ((x[2][0] + x[2][1]) + (x[2][2] + x[2][3])) + ((x[3][0] + x[3][1]) + (x[3][2] + x[3][3]));
+            s += dpp_get<kDppXor1>(s);
         }
-        // fold the tpr (2, 4, 8 or 16) neighbouring lanes; every lane ends with the total
-        float o = dpp_get<kDppXor1>(s);
-        s = MAX ? fmaxf(s, o) : s + o;
-        if (tpr >= 4) { o = dpp_get<kDppXor2>(s); s = MAX ? fmaxf(s, o) : s + o; }
-        if (tpr >= 8) { o = dpp_get<kDppHalfMirror>(s); s = MAX ? fmaxf(s, o) : s + o; }
-        if (tpr >= 16) { o = dpp_get<kDppMirror>(s); s = MAX ? fmaxf(s, o) : s + o; }
-        const float res = post(row, s);
-        if (sub == 0) row_out[row] = res;
     }
+    // waves: one partial per (row, key group), dense so that 256 floats cover the workgroup
+    float *part = rr.part + (rr.parity & 1) * 256;
+    rr.parity ^= 1;
+    const int pbase = (qg * 32 + row) * kg_n;
+    if (half == 0) part[pbase + kg] = s;
     __syncthreads();
+    float tot = part[pbase];
+    if (kg_n > 1) tot = MAX ? fmaxf(tot, part[pbase + 1]) : tot + part[pbase + 1];
+    if (kg_n > 2) {
+        const float t2 = part[pbase + 2], t3 = part[pbase + 3];
+        tot = MAX ? fmaxf(tot, fmaxf(t2, t3)) : tot + (t2 + t3);
+    }
+    if (kg_n > 4) {
+        const float t4 = part[pbase + 4], t5 = part[pbase + 5], t6 = part[pbase + 6], t7 = part[pbase + 7];
+        tot = MAX ? fmaxf(tot, fmaxf(fmaxf(t4, t5), fmaxf(t6, t7))) : tot + ((t4 + t5) + (t6 + t7));
+    }
+    bool out_of_range = false;
+    if (!MAX) {
+        // every wave looks at all 256 partials of the workgroup: lane L at floats [4L, 4L + 4)
+        const floatx4 f = reinterpret_cast<const floatx4 *>(part)[lane];
+        const bool hi = !(f[0] < kSumHi) || !(f[1] < kSumHi) || !(f[2] < kSumHi) || !(f[3] < kSumHi);
+        const float m01 = fmaxf(f[0], f[1]), m23 = fmaxf(f[2], f[3]);
+        float lowest;  // smallest per-row maximum over key groups among the rows this lane sees
+        if (kg_n >= 4) {
+            lowest = fmaxf(m01, m23);
+            if (kg_n == 8) lowest = fmaxf(lowest, dpp_get<kDppXor1>(lowest));
+        } else if (kg_n == 2) {
+            lowest = fminf(m01, m23);
+        } else {
+            lowest = fminf(fminf(f[0], f[1]), fminf(f[2], f[3]));
+        }
+        out_of_range = __builtin_amdgcn_ballot_w64(hi || !(lowest >= kSumLo)) != 0;
+    }
+    const float res = post(qg * 32 + row, tot);
+    if (half == 0) rr.wv_w[row] = res;
+    __builtin_amdgcn_wave_barrier();
+    return out_of_range;
+}
+
+// the four values of rows 8*i4 + 4*g + {0..3} left by reduce_rows
+__device__ __forceinline__ floatx4 row_values(const RowRed &rr, int i4, int g)
+{
+    return *reinterpret_cast<const floatx4 *>(rr.wv_w + 8 * i4 + 4 * g);
 }
 
 }  // namespace
-
-#define FCS_GLDS16(gptr, lptr)                                                                   \
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gptr),    \
-                                     (__attribute__((address_space(3))) void *)(lptr), 16, 0, 0)
-#define FCS_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
-// stops the compiler from precomputing per-tile values of a scalar for the whole walk
-#define FCS_OPAQUE_S(x) asm volatile("" : "+s"(x))
-#define FCS_OPAQUE_V(x) asm volatile("" : "+v"(x))
 
 // RAGGED = false: S_k is exactly (key groups) x TPW x 32, no padding keys anywhere.
 // RAGGED = true : the last tiles may hold padding keys; every exponent is masked per lane.
@@ -95,10 +144,11 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     constexpr int AHEAD = NS - 1;          // items in flight ahead of the one being consumed
     constexpr int ITEMS = TPW + 1;         // per (head, row block): the Q tile, then TPW key tiles
     constexpr int SLOT_BYTES = NT * 1024;  // one item: NT pieces x 64 lanes x 16 bytes
-    __shared__ __attribute__((aligned(16))) float red[8192];
-    __shared__ __attribute__((aligned(16))) float rowv[256];
+    constexpr bool STATIC_SLOTS = (ITEMS % NS == 0);  // then item j of every head sits in slot j % NS
     __shared__ __attribute__((aligned(16))) char ring[8 * NS * SLOT_BYTES];
-    __shared__ int redo[2];
+    __shared__ __attribute__((aligned(16))) float red[8 * 32 * kRedPitch];
+    __shared__ __attribute__((aligned(16))) float part[2 * 256];
+    __shared__ __attribute__((aligned(16))) float wv[8 * 32];
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what derives from it stays in SGPRs
@@ -114,8 +164,11 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     const int k_full = max(0, min(TPW, (a.Sk - kbase) / 32));  // key tiles of this wave without padding keys
     const bool q_full = (q0 + 32 <= a.Sq);
 
-    if (tid < 2) redo[tid] = 0;
-    __syncthreads();
+    RowRed rr;
+    rr.red_w = red + wave * (32 * kRedPitch);
+    rr.part = part;
+    rr.wv_w = wv + wave * 32;
+    rr.parity = 0;
 
     // Operand tiles are 32 rows x 64 halves (128 B per row).  One DMA instruction moves 8
     // whole rows (1 KB, 8 full cache lines): lane L brings 16-byte piece L % 8 of row L / 8,
@@ -124,7 +177,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // the pieces of a row are stored XOR-swizzled: position p of row r holds piece
     // p ^ ((r >> 1) & 7).  The swizzle only depends on the parity of the instruction index.
     int lrow = lane >> 3;  // row within the 8 rows of one DMA instruction
-    uint32_t piece_b[2];         // byte offset in its row of the piece this lane fetches (even / odd instruction)
+    uint32_t piece_b[2];   // byte offset in its row of the piece this lane fetches (even / odd instruction)
 #pragma unroll
     for (int par = 0; par < 2; ++par) piece_b[par] = (uint32_t)(((lane & 7) ^ ((par * 4 + (lane >> 4)) & 7)) * 16);
     const uint32_t q_row_b = (uint32_t)a.qs_s * 2u, k_row_b = (uint32_t)a.ks_s * 2u;  // row pitch in bytes
@@ -135,23 +188,31 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     const int64_t q_head_b = a.qs_h * 2, k_head_b = a.ks_h * 2;
     char *my_ring = ring + wave * (NS * SLOT_BYTES);
 
-    // DMA rows [0, 32) of the tile starting at `tile` (uniform) into ring slot `slot`.
-    // `rows_left` <= 31 marks a tile that runs past the end of its tensor slice: such rows are
-    // replaced by the last real row (they are masked or ignored by the consumer).
-    auto fetch_tile = [&](const char *tile, uint32_t row_b, const uint32_t (&voff)[2], bool full, int rows_left, int slot) {
+    // DMA rows [0, 32) of the tile starting at `tile` (wave-uniform) into ring slot `slot`.
+    // Not `full`: the tile runs past the end of its tensor slice after `rows_left` rows; those
+    // rows are replaced by the last real row (the consumer masks or ignores them).
+    auto fetch_tile = [&](const char *tile, uint32_t row_b, uint32_t (&voff)[2], bool full, int rows_left, int slot) {
         char *dst = my_ring + slot * SLOT_BYTES;
         if (full) {
-#pragma unroll
-            for (int tt = 0; tt < NT; ++tt) FCS_GLDS16(tile + (uint32_t)(tt * 8) * row_b + voff[tt & 1], dst + tt * 1024);
-        } else {
+            FCS_OPAQUE_V(voff[0]);
+            FCS_OPAQUE_V(voff[1]);
 #pragma unroll
             for (int tt = 0; tt < NT; ++tt) {
-                const int row = max(0, min(tt * 8 + lrow, rows_left - 1));
-                FCS_GLDS16(tile + (uint32_t)row * row_b + piece_b[tt & 1], dst + tt * 1024);
+                const char *rows8 = tile + (size_t)((uint32_t)(tt * 8) * row_b);  // scalar base + 32-bit lane offset
+                FCS_GLDS16(rows8 + voff[tt & 1], dst + tt * 1024);
+            }
+        } else {
+            FCS_OPAQUE_V(lrow);
+            FCS_OPAQUE_V(piece_b[0]);
+            FCS_OPAQUE_V(piece_b[1]);
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) {
+                const uint32_t row = (uint32_t)max(0, min(tt * 8 + lrow, rows_left - 1));
+                FCS_GLDS16(tile + (row * row_b + piece_b[tt & 1]), dst + tt * 1024);
             }
         }
     };
-    // read a ring slot back as an MFMA operand: lane (n, g) takes, for step tt, piece 2*tt + g of
+    // Read a ring slot back as an MFMA operand: lane (n, g) takes, for step tt, piece 2*tt + g of
     // row n.  Issued from inline assembly: the compiler would otherwise make every LDS read wait
     // for ALL outstanding DMA fetches (vmcnt(0)), which would undo the look-ahead.
     uint32_t take_addr[NT];
@@ -159,15 +220,26 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     for (int tt = 0; tt < NT; ++tt)
         take_addr[tt] = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)my_ring +
                         (uint32_t)(n * 128 + (((2 * tt + g) ^ ((n >> 1) & 7)) * 16));
+    static_assert(NT == 4 && SLOT_BYTES == 4096, "the operand reads below are written for four 1 KB pieces");
+#define FCS_TAKE_ASM(OFF)                                                                                        \
+    asm volatile("ds_read_b128 %0, %4 offset:" #OFF "\n\tds_read_b128 %1, %5 offset:" #OFF                     \
+                 "\n\tds_read_b128 %2, %6 offset:" #OFF "\n\tds_read_b128 %3, %7 offset:" #OFF "\n\ts_waitcnt lgkmcnt(0)" \
+                 : "=&v"(dst[0]), "=&v"(dst[1]), "=&v"(dst[2]), "=&v"(dst[3])                                  \
+                 : "v"(ta0), "v"(ta1), "v"(ta2), "v"(ta3)                                                       \
+                 : "memory")
     auto take = [&](int slot, half8 (&dst)[NT]) {
-        const uint32_t off = (uint32_t)(slot * SLOT_BYTES);
-        static_assert(NT == 4, "four pieces per lane");
-        asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7\n\t"
-                     "s_waitcnt lgkmcnt(0)"
-                     : "=&v"(dst[0]), "=&v"(dst[1]), "=&v"(dst[2]), "=&v"(dst[3])
-                     : "v"(take_addr[0] + off), "v"(take_addr[1] + off), "v"(take_addr[2] + off), "v"(take_addr[3] + off)
-                     : "memory");
+        if (STATIC_SLOTS) {  // slot is a compile-time value at every call site: it folds into the offset field
+            const uint32_t ta0 = take_addr[0], ta1 = take_addr[1], ta2 = take_addr[2], ta3 = take_addr[3];
+            if (slot == 0) FCS_TAKE_ASM(0);
+            else if (slot == 1) FCS_TAKE_ASM(4096);
+            else FCS_TAKE_ASM(8192);
+        } else {
+            const uint32_t off = (uint32_t)(slot * SLOT_BYTES);
+            const uint32_t ta0 = take_addr[0] + off, ta1 = take_addr[1] + off, ta2 = take_addr[2] + off, ta3 = take_addr[3] + off;
+            FCS_TAKE_ASM(0);
+        }
     };
+#undef FCS_TAKE_ASM
 
     float col_acc[TPW];
 #pragma unroll
@@ -177,32 +249,27 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // ring slot i % NS; while item i is consumed, item i + AHEAD is fetched into the slot that
     // item i - 1 just left.  Past the last head the fetches repeat it, so that the number of
     // outstanding DMA instructions at every wait is a compile-time constant.
-    auto fetch_item = [&](const char *qh, const char *kh, int j, int slot) {  // j: position in the head, compile-time
+    auto fetch_item = [&](const char *qh, const char *kh, int j /* position in the head, compile-time */, int slot) {
         if (j == 0)
             fetch_tile(qh, q_row_b, q_voff, q_full, a.Sq - q0, slot);
         else
-            fetch_tile(kh + (int64_t)((j - 1) * 32) * k_row_b, k_row_b, k_voff, (j - 1) < k_full, a.Sk - kbase - (j - 1) * 32, slot);
+            fetch_tile(kh + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff, (j - 1) < k_full,
+                       a.Sk - kbase - (j - 1) * 32, slot);
     };
 
-    int cs = 0;  // slot of the item being consumed
+    int cs = 0;  // slot of the item being consumed (when the slots are not static)
     {
+        const int h1 = min(h_begin + 1, h_end - 1);
         const char *qh = q_b + (int64_t)h_begin * q_head_b, *kh = k_b + (int64_t)h_begin * k_head_b;
-        const char *qh1 = q_b + (int64_t)min(h_begin + 1, h_end - 1) * q_head_b, *kh1 = k_b + (int64_t)min(h_begin + 1, h_end - 1) * k_head_b;
+        const char *qh1 = q_b + (int64_t)h1 * q_head_b, *kh1 = k_b + (int64_t)h1 * k_head_b;
 #pragma unroll
         for (int i = 0; i < AHEAD; ++i) fetch_item(i < ITEMS ? qh : qh1, i < ITEMS ? kh : kh1, i % ITEMS, i % NS);
     }
 
     for (int unit = 0; unit < n_units; ++unit) {
-        // pointers of this head and of the next one (the last head repeats); kept opaque so that
-        // per-tile addresses are formed when needed instead of being held in registers
-        const int h = h_begin + unit, h1 = min(h + 1, h_end - 1);
+        const int h = h_begin + unit, h1 = min(h + 1, h_end - 1);  // the last head repeats
         const char *qh = q_b + (int64_t)h * q_head_b, *kh = k_b + (int64_t)h * k_head_b;
         const char *qh1 = q_b + (int64_t)h1 * q_head_b, *kh1 = k_b + (int64_t)h1 * k_head_b;
-        uint32_t k_row_b_o = k_row_b;
-        FCS_OPAQUE_S(k_row_b_o);
-        (void)k_row_b_o;
-        FCS_OPAQUE_V(q_voff[0]); FCS_OPAQUE_V(q_voff[1]); FCS_OPAQUE_V(k_voff[0]); FCS_OPAQUE_V(k_voff[1]);
-        FCS_OPAQUE_V(piece_b[0]); FCS_OPAQUE_V(piece_b[1]); FCS_OPAQUE_V(lrow);
 
         floatx16 acc[TPW];
         float rs[16];
@@ -232,11 +299,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         auto step = [&](int j, half8 (&dst)[NT]) {
             const int fj = (j + AHEAD) % ITEMS;
             const bool next_head = (j + AHEAD) >= ITEMS;
-            const int fs = (cs == 0) ? NS - 1 : cs - 1;  // the slot item (this - 1) just left
+            const int here = STATIC_SLOTS ? j % NS : cs;
+            const int fs = (here == 0) ? NS - 1 : here - 1;  // the slot item (this - 1) just left
             fetch_item(next_head ? qh1 : qh, next_head ? kh1 : kh, fj, fs);
             FCS_WAIT_VM(AHEAD * NT);
-            take(cs, dst);
-            cs = (cs == NS - 1) ? 0 : cs + 1;
+            take(here, dst);
+            if (!STATIC_SLOTS) cs = (cs == NS - 1) ? 0 : cs + 1;
         };
 
         // ---------------- phase 1
@@ -254,18 +322,21 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 #pragma unroll
             for (int tt = 0; tt < NT; ++tt) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[tt], kf[tt], c, 0, 0, 0);
             acc[t] = c;
-            if (t > 0) exp_tile(t - 1);  // VALU work of the previous tile runs under this tile's MFMAs
+            if (t > 0) {
+                // VALU work of the previous tile runs under this tile's MFMAs.  The row sums are
+                // pinned here: otherwise the optimiser sinks every exponent below the last MFMA.
+                exp_tile(t - 1);
+                asm volatile("" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]), "+v"(rs[4]), "+v"(rs[5]), "+v"(rs[6]),
+                             "+v"(rs[7]), "+v"(rs[8]), "+v"(rs[9]), "+v"(rs[10]), "+v"(rs[11]), "+v"(rs[12]), "+v"(rs[13]),
+                             "+v"(rs[14]), "+v"(rs[15]));
+            }
         }
         exp_tile(TPW - 1);
 
         // ---------------- row sums over lanes and key-group waves; w = 1/L (0 for rows not averaged)
-        int *flag = &redo[unit & 1];
-        reduce_rows<false>(rs, red, rowv, kg_n, qg, kg, n, g, tid, [&](int row, float L) {
-            if (!(L >= kSumLo && L < kSumHi)) *flag = 1;
+        const bool slow = reduce_rows<false>(rs, rr, kg_n, qg, kg, lane, [&](int row, float L) {
             return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
         });
-        const bool slow = (*flag != 0);
-        if (tid == 0) redo[(unit + 1) & 1] = 0;
 
         if (slow) {
             // ------------ rare: max-subtracted softmax for this (head, row block).  Operands are
@@ -293,12 +364,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) rs[i] = fmaxf(rs[i], real ? c[i] : kNegBig);
             }
-            reduce_rows<true>(rs, red, rowv, kg_n, qg, kg, n, g, tid, [&](int, float m) { return m; });
+            reduce_rows<true>(rs, rr, kg_n, qg, kg, lane, [&](int, float m) { return m; });
 #pragma unroll
             for (int i = 0; i < 16; ++i) rs[i] = 0.f;
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
-                const floatx4 m4 = *reinterpret_cast<const floatx4 *>(&rowv[qg * 32 + 8 * i4 + 4 * g]);
+                const floatx4 m4 = row_values(rr, i4, g);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const float nm = -m4[j] * a.c;
@@ -311,7 +382,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                     }
                 }
             }
-            reduce_rows<false>(rs, red, rowv, kg_n, qg, kg, n, g, tid, [&](int row, float L) {
+            reduce_rows<false>(rs, rr, kg_n, qg, kg, lane, [&](int row, float L) {
                 return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
             });
         }
@@ -319,7 +390,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         // ---------------- phase 3: column sums of e * w
 #pragma unroll
         for (int i4 = 0; i4 < 4; ++i4) {
-            const floatx4 w4 = *reinterpret_cast<const floatx4 *>(&rowv[qg * 32 + 8 * i4 + 4 * g]);
+            const floatx4 w4 = row_values(rr, i4, g);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
 #pragma unroll
