@@ -133,8 +133,10 @@ __device__ __forceinline__ floatx4 row_values(const RowRed &rr, int i4, int g)
 
 }  // namespace
 
-// RAGGED = false: S_k is exactly (key groups) x TPW x 32, no padding keys anywhere.
-// RAGGED = true : the last tiles may hold padding keys; every exponent is masked per lane.
+// RAGGED = false: S_k is exactly (key groups) x TPW x 32 and S_q a multiple of the block's rows:
+//                 every operand tile is whole, no padding keys anywhere.
+// RAGGED = true : tiles may run past the tensors; fetches clamp their rows and every exponent is
+//                 masked per lane.
 template <int D, int TPW, bool RAGGED>
 __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 {
@@ -161,8 +163,6 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     const int blk_row0 = qblk * 32 * qg_n;  // first query row of the block
     const int q0 = blk_row0 + qg * 32;      // first query row of this wave
     const int kbase = kg * TPW * 32;        // first key of this wave
-    const int k_full = max(0, min(TPW, (a.Sk - kbase) / 32));  // key tiles of this wave without padding keys
-    const bool q_full = (q0 + 32 <= a.Sq);
 
     RowRed rr;
     rr.red_w = red + wave * (32 * kRedPitch);
@@ -188,46 +188,41 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     const int64_t q_head_b = a.qs_h * 2, k_head_b = a.ks_h * 2;
     char *my_ring = ring + wave * (NS * SLOT_BYTES);
 
-    // DMA rows [0, 32) of the tile starting at `tile` (wave-uniform) into ring slot `slot`.
-    // Not `full`: the tile runs past the end of its tensor slice after `rows_left` rows; those
-    // rows are replaced by the last real row (the consumer masks or ignores them).
-    auto fetch_tile = [&](const char *tile, uint32_t row_b, uint32_t (&voff)[2], bool full, int rows_left, int slot) {
-        char *dst = my_ring + slot * SLOT_BYTES;
-        if (full) {
-            FCS_OPAQUE_V(voff[0]);
-            FCS_OPAQUE_V(voff[1]);
-#pragma unroll
-            for (int tt = 0; tt < NT; ++tt) {
-                const char *rows8 = tile + (size_t)((uint32_t)(tt * 8) * row_b);  // scalar base + 32-bit lane offset
-                FCS_GLDS16(rows8 + voff[tt & 1], dst + tt * 1024);
-            }
+    // DMA instruction `tt` (of NT) of a tile: rows [8*tt, 8*tt + 8) of the tile starting at `tile`
+    // (wave-uniform) go to ring slot `slot`.  In the ragged kernel a tile may run past the end of
+    // its tensor slice after `rows_left` rows; those rows are replaced by the last real row (the
+    // consumer masks or ignores them).  No branch either way: a taken branch costs a wave far
+    // more than the few address instructions it would skip.
+    auto fetch_piece = [&](const char *tile, uint32_t row_b, uint32_t (&voff)[2], int rows_left, int slot, int tt) {
+        char *dst = my_ring + slot * SLOT_BYTES + tt * 1024;
+        if (!RAGGED) {  // every tile is whole: scalar base + one 32-bit lane offset, no branch
+            FCS_OPAQUE_V(voff[tt & 1]);
+            const char *rows8 = tile + (size_t)((uint32_t)(tt * 8) * row_b);
+            FCS_GLDS16(rows8 + voff[tt & 1], dst);
         } else {
             FCS_OPAQUE_V(lrow);
-            FCS_OPAQUE_V(piece_b[0]);
-            FCS_OPAQUE_V(piece_b[1]);
-#pragma unroll
-            for (int tt = 0; tt < NT; ++tt) {
-                const uint32_t row = (uint32_t)max(0, min(tt * 8 + lrow, rows_left - 1));
-                FCS_GLDS16(tile + (row * row_b + piece_b[tt & 1]), dst + tt * 1024);
-            }
+            FCS_OPAQUE_V(piece_b[tt & 1]);
+            const uint32_t row = (uint32_t)max(0, min(tt * 8 + lrow, rows_left - 1));
+            FCS_GLDS16(tile + (row * row_b + piece_b[tt & 1]), dst);
         }
     };
     // Read a ring slot back as an MFMA operand: lane (n, g) takes, for step tt, piece 2*tt + g of
     // row n.  Issued from inline assembly: the compiler would otherwise make every LDS read wait
-    // for ALL outstanding DMA fetches (vmcnt(0)), which would undo the look-ahead.
+    // for ALL outstanding DMA fetches (vmcnt(0)), which would undo the look-ahead.  The reads
+    // are only ISSUED here; take_wait() must sit between them and the first use of `dst`.
     uint32_t take_addr[NT];
 #pragma unroll
     for (int tt = 0; tt < NT; ++tt)
         take_addr[tt] = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)my_ring +
                         (uint32_t)(n * 128 + (((2 * tt + g) ^ ((n >> 1) & 7)) * 16));
     static_assert(NT == 4 && SLOT_BYTES == 4096, "the operand reads below are written for four 1 KB pieces");
-#define FCS_TAKE_ASM(OFF)                                                                                        \
-    asm volatile("ds_read_b128 %0, %4 offset:" #OFF "\n\tds_read_b128 %1, %5 offset:" #OFF                     \
-                 "\n\tds_read_b128 %2, %6 offset:" #OFF "\n\tds_read_b128 %3, %7 offset:" #OFF "\n\ts_waitcnt lgkmcnt(0)" \
-                 : "=&v"(dst[0]), "=&v"(dst[1]), "=&v"(dst[2]), "=&v"(dst[3])                                  \
-                 : "v"(ta0), "v"(ta1), "v"(ta2), "v"(ta3)                                                       \
+#define FCS_TAKE_ASM(OFF)                                                                                  \
+    asm volatile("ds_read_b128 %0, %4 offset:" #OFF "\n\tds_read_b128 %1, %5 offset:" #OFF                 \
+                 "\n\tds_read_b128 %2, %6 offset:" #OFF "\n\tds_read_b128 %3, %7 offset:" #OFF             \
+                 : "=&v"(dst[0]), "=&v"(dst[1]), "=&v"(dst[2]), "=&v"(dst[3])                              \
+                 : "v"(ta0), "v"(ta1), "v"(ta2), "v"(ta3)                                                   \
                  : "memory")
-    auto take = [&](int slot, half8 (&dst)[NT]) {
+    auto take_issue = [&](int slot, half8 (&dst)[NT]) {
         if (STATIC_SLOTS) {  // slot is a compile-time value at every call site: it folds into the offset field
             const uint32_t ta0 = take_addr[0], ta1 = take_addr[1], ta2 = take_addr[2], ta3 = take_addr[3];
             if (slot == 0) FCS_TAKE_ASM(0);
@@ -240,37 +235,55 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         }
     };
 #undef FCS_TAKE_ASM
+    // all LDS reads issued so far have landed; ties the operand registers so that no use moves above
+    auto take_wait = [&](half8 (&dst)[NT]) {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(dst[0]), "+v"(dst[1]), "+v"(dst[2]), "+v"(dst[3])::"memory");
+    };
 
     float col_acc[TPW];
 #pragma unroll
     for (int t = 0; t < TPW; ++t) col_acc[t] = 0.f;
 
-    // The walk: for every head the Q tile, then the TPW key tiles ("items").  Item i lives in
-    // ring slot i % NS; while item i is consumed, item i + AHEAD is fetched into the slot that
-    // item i - 1 just left.  Past the last head the fetches repeat it, so that the number of
-    // outstanding DMA instructions at every wait is a compile-time constant.
-    auto fetch_item = [&](const char *qh, const char *kh, int j /* position in the head, compile-time */, int slot) {
+    // The walk.  Every head contributes ITEMS = 1 + TPW operand tiles ("items"): its Q tile, then
+    // the wave's key tiles.  Item number p (counted over the whole walk) lives in ring slot p % 3.
+    //   * Items are read back into registers ONE STEP BEFORE the MFMAs that use them, so the LDS
+    //     latency is covered by the exponent work of the step in between.
+    //   * As soon as the read-back of item p has landed its slot is free, and item p + 3 is
+    //     fetched into it; at most three items (12 DMA instructions) are in flight.
+    //   * Past the last head the fetches repeat it, so that the number of outstanding DMA
+    //     instructions at every wait is a compile-time constant.
+    auto fetch_pos_piece = [&](int h_now, int j_ahead /* item index counted from the Q tile of head h_now, compile-time */,
+                               int slot, int tt) {
+        const int hh = min(h_now + j_ahead / ITEMS, h_end - 1);
+        const int j = j_ahead % ITEMS;
         if (j == 0)
-            fetch_tile(qh, q_row_b, q_voff, q_full, a.Sq - q0, slot);
+            fetch_piece(q_b + (int64_t)hh * q_head_b, q_row_b, q_voff, a.Sq - q0, slot, tt);
         else
-            fetch_tile(kh + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff, (j - 1) < k_full,
-                       a.Sk - kbase - (j - 1) * 32, slot);
+            fetch_piece(k_b + (int64_t)hh * k_head_b + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff,
+                        a.Sk - kbase - (j - 1) * 32, slot, tt);
+    };
+    auto fetch_pos = [&](int h_now, int j_ahead, int slot) {
+#pragma unroll
+        for (int tt = 0; tt < NT; ++tt) fetch_pos_piece(h_now, j_ahead, slot, tt);
+    };
+    int sq = 0;  // ring slot of the current head's Q tile (only used when the slots are not static)
+    auto slot_of = [&](int j) {  // slot of item j of the current head, j compile-time, j < ITEMS + 3
+        if (STATIC_SLOTS) return j % NS;
+        int s_ = sq + (j % NS);
+        return s_ >= NS ? s_ - NS : s_;
     };
 
-    int cs = 0;  // slot of the item being consumed (when the slots are not static)
-    {
-        const int h1 = min(h_begin + 1, h_end - 1);
-        const char *qh = q_b + (int64_t)h_begin * q_head_b, *kh = k_b + (int64_t)h_begin * k_head_b;
-        const char *qh1 = q_b + (int64_t)h1 * q_head_b, *kh1 = k_b + (int64_t)h1 * k_head_b;
+    half8 qf[NT], kf[2][NT];
 #pragma unroll
-        for (int i = 0; i < AHEAD; ++i) fetch_item(i < ITEMS ? qh : qh1, i < ITEMS ? kh : kh1, i % ITEMS, i % NS);
-    }
+    for (int i = 0; i < NS; ++i) fetch_pos(h_begin, i, i);
 
     for (int unit = 0; unit < n_units; ++unit) {
-        const int h = h_begin + unit, h1 = min(h + 1, h_end - 1);  // the last head repeats
-        const char *qh = q_b + (int64_t)h * q_head_b, *kh = k_b + (int64_t)h * k_head_b;
-        const char *qh1 = q_b + (int64_t)h1 * q_head_b, *kh1 = k_b + (int64_t)h1 * k_head_b;
-
+        const int h = h_begin + unit;
+        // this head's Q tile and first key tile (fetched during the previous head)
+        FCS_WAIT_VM(2 * NT);
+        take_issue(slot_of(0), qf);
+        FCS_WAIT_VM(1 * NT);
+        take_issue(slot_of(1), kf[0]);
         floatx16 acc[TPW];
         float rs[16];
 #pragma unroll
@@ -278,123 +291,142 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 
         // e = 2^(c*s) for tile t, in place, and its contribution to the row sums
         auto exp_tile = [&](int t) {
-            if (!RAGGED) {
+            const bool real = !RAGGED || (kbase + t * 32 + n) < a.Sk;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float e = fast_exp2(acc[t][i] * a.c);
-                    acc[t][i] = e;
-                    rs[i] += e;
-                }
-            } else {
-                const bool real = (kbase + t * 32 + n) < a.Sk;
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float e = real ? fast_exp2(acc[t][i] * a.c) : 0.f;
-                    acc[t][i] = e;
-                    rs[i] += e;
-                }
+            for (int i = 0; i < 16; ++i) {
+                const float e = real ? fast_exp2(acc[t][i] * a.c) : 0.f;
+                acc[t][i] = e;
+                rs[i] += e;
             }
-        };
-        // one step of the walk: start the look-ahead fetch, wait for this item, read it back
-        auto step = [&](int j, half8 (&dst)[NT]) {
-            const int fj = (j + AHEAD) % ITEMS;
-            const bool next_head = (j + AHEAD) >= ITEMS;
-            const int here = STATIC_SLOTS ? j % NS : cs;
-            const int fs = (here == 0) ? NS - 1 : here - 1;  // the slot item (this - 1) just left
-            fetch_item(next_head ? qh1 : qh, next_head ? kh1 : kh, fj, fs);
-            FCS_WAIT_VM(AHEAD * NT);
-            take(here, dst);
-            if (!STATIC_SLOTS) cs = (cs == NS - 1) ? 0 : cs + 1;
+            // pinned here: otherwise the optimiser sinks every exponent below the last MFMA
+            asm volatile("" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]), "+v"(rs[4]), "+v"(rs[5]), "+v"(rs[6]),
+                         "+v"(rs[7]), "+v"(rs[8]), "+v"(rs[9]), "+v"(rs[10]), "+v"(rs[11]), "+v"(rs[12]), "+v"(rs[13]),
+                         "+v"(rs[14]), "+v"(rs[15]));
         };
 
-        // ---------------- phase 1
-        half8 qf[NT];
-        step(0, qf);
-        if (a.negate) {
-#pragma unroll
-            for (int tt = 0; tt < NT; ++tt) qf[tt] = flip_sign(qf[tt]);
-        }
+        // ---------------- phase 1: one step per key tile
 #pragma unroll
         for (int t = 0; t < TPW; ++t) {
-            half8 kf[NT];
-            step(1 + t, kf);
+            // the operands of this tile were read back during the previous step: they have landed,
+            // their ring slots are free again and take the look-ahead fetches
+            if (t == 0) {
+                take_wait(qf);
+                take_wait(kf[0]);
+                if (a.negate) {
+#pragma unroll
+                    for (int tt = 0; tt < NT; ++tt) qf[tt] = flip_sign(qf[tt]);
+                }
+                fetch_pos(h, 0 + NS, slot_of(0));
+                fetch_pos(h, 1 + NS, slot_of(1));
+            } else {
+                take_wait(kf[t & 1]);
+                fetch_pos(h, 1 + t + NS, slot_of(1 + t));
+            }
+            FCS_WAIT_VM(2 * NT);  // the next key tile has landed; two later items may be in flight
+            if (t + 1 < TPW) take_issue(slot_of(2 + t), kf[(t + 1) & 1]);
             floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int tt = 0; tt < NT; ++tt) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[tt], kf[tt], c, 0, 0, 0);
+            for (int tt = 0; tt < NT; ++tt) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[tt], kf[t & 1][tt], c, 0, 0, 0);
             acc[t] = c;
-            if (t > 0) {
-                // VALU work of the previous tile runs under this tile's MFMAs.  The row sums are
-                // pinned here: otherwise the optimiser sinks every exponent below the last MFMA.
-                exp_tile(t - 1);
-                asm volatile("" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]), "+v"(rs[4]), "+v"(rs[5]), "+v"(rs[6]),
-                             "+v"(rs[7]), "+v"(rs[8]), "+v"(rs[9]), "+v"(rs[10]), "+v"(rs[11]), "+v"(rs[12]), "+v"(rs[13]),
-                             "+v"(rs[14]), "+v"(rs[15]));
-            }
+            if (t > 0) exp_tile(t - 1);  // VALU work of the previous tile runs under this tile's MFMAs
         }
         exp_tile(TPW - 1);
+
+        if (!STATIC_SLOTS) {
+            sq += ITEMS % NS;
+            if (sq >= NS) sq -= NS;
+        }
 
         // ---------------- row sums over lanes and key-group waves; w = 1/L (0 for rows not averaged)
         const bool slow = reduce_rows<false>(rs, rr, kg_n, qg, kg, lane, [&](int row, float L) {
             return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
         });
 
-        if (slow) {
-            // ------------ rare: max-subtracted softmax for this (head, row block).  Operands are
-            // fetched again with ordinary loads (the ring keeps streaming ahead untouched).
-            const _Float16 *qp = reinterpret_cast<const _Float16 *>(qh) + (int64_t)min(n, a.Sq - 1 - q0) * a.qs_s + g * 8;
-            const _Float16 *kp = reinterpret_cast<const _Float16 *>(kh) + g * 8;
+        if (!slow) {
+            // ---------------- phase 3: column sums of e * w
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const floatx4 w4 = row_values(rr, i4, g);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int t = 0; t < TPW; ++t) col_acc[t] = fmaf(acc[t][4 * i4 + j], w4[j], col_acc[t]);
+                }
+            }
+        } else {
+            // ------------ rare: max-subtracted softmax for this (head, row block), three passes over
+            // the keys with one score tile in registers at a time.  Operands come through ordinary
+            // loads; the ring and the operands already read back for the next head are untouched.
+            // lane-dependent values are rebuilt here from an opaque copy of the lane id, so that
+            // nothing of this rare path is precomputed and kept in registers by the common path
+            int lane_s = lane;
+            FCS_OPAQUE_V(lane_s);
+            const int n_s = lane_s & 31, g_s = lane_s >> 5;
+            const _Float16 *qp = reinterpret_cast<const _Float16 *>(q_b + (int64_t)h * q_head_b) +
+                                 (int64_t)min(n_s, a.Sq - 1 - q0) * a.qs_s + g_s * 8;
+            const _Float16 *kp = reinterpret_cast<const _Float16 *>(k_b + (int64_t)h * k_head_b) + g_s * 8;
+            half8 qs[NT];
 #pragma unroll
             for (int tt = 0; tt < NT; ++tt) {
                 const half8 v = load8(qp + tt * 16);
-                qf[tt] = a.negate ? flip_sign(v) : v;
+                qs[tt] = a.negate ? flip_sign(v) : v;
             }
+            auto score_tile = [&](int t) {
+                half8 ks[NT];
+                const int krow = max(0, min(t * 32 + n_s, a.Sk - 1 - kbase));
 #pragma unroll
-            for (int i = 0; i < 16; ++i) rs[i] = kNegBig;
-#pragma unroll
-            for (int t = 0; t < TPW; ++t) {
-                half8 kf[NT];
-                const int krow = max(0, min(t * 32 + n, a.Sk - 1 - kbase));
-#pragma unroll
-                for (int tt = 0; tt < NT; ++tt) kf[tt] = load8(kp + (int64_t)krow * a.ks_s + tt * 16);
+                for (int tt = 0; tt < NT; ++tt) ks[tt] = load8(kp + (int64_t)krow * a.ks_s + tt * 16);
                 floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int tt = 0; tt < NT; ++tt) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[tt], kf[tt], c, 0, 0, 0);
-                acc[t] = c;
-                const bool real = (kbase + t * 32 + n) < a.Sk;
+                for (int tt = 0; tt < NT; ++tt) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(qs[tt], ks[tt], c, 0, 0, 0);
+                return c;
+            };
+            float v16[16];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) rs[i] = fmaxf(rs[i], real ? c[i] : kNegBig);
+            for (int i = 0; i < 16; ++i) v16[i] = kNegBig;
+#pragma unroll 1
+            for (int t = 0; t < TPW; ++t) {
+                const floatx16 c = score_tile(t);
+                const bool real = (kbase + t * 32 + n_s) < a.Sk;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v16[i] = fmaxf(v16[i], real ? c[i] : kNegBig);
             }
-            reduce_rows<true>(rs, rr, kg_n, qg, kg, lane, [&](int, float m) { return m; });
-#pragma unroll
-            for (int i = 0; i < 16; ++i) rs[i] = 0.f;
+            reduce_rows<true>(v16, rr, kg_n, qg, kg, lane_s, [&](int, float m) { return m; });
+            float nm[16];
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
-                const floatx4 m4 = row_values(rr, i4, g);
+                const floatx4 m4 = row_values(rr, i4, g_s);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float nm = -m4[j] * a.c;
-#pragma unroll
-                    for (int t = 0; t < TPW; ++t) {
-                        const bool real = (kbase + t * 32 + n) < a.Sk;
-                        const float e = real ? fast_exp2(fmaf(acc[t][4 * i4 + j], a.c, nm)) : 0.f;
-                        acc[t][4 * i4 + j] = e;
-                        rs[4 * i4 + j] += e;
-                    }
-                }
+                for (int j = 0; j < 4; ++j) nm[4 * i4 + j] = -m4[j] * a.c;
             }
-            reduce_rows<false>(rs, rr, kg_n, qg, kg, lane, [&](int row, float L) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v16[i] = 0.f;
+#pragma unroll 1
+            for (int t = 0; t < TPW; ++t) {
+                const floatx16 c = score_tile(t);
+                const bool real = (kbase + t * 32 + n_s) < a.Sk;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v16[i] += real ? fast_exp2(fmaf(c[i], a.c, nm[i])) : 0.f;
+            }
+            reduce_rows<false>(v16, rr, kg_n, qg, kg, lane_s, [&](int row, float L) {
                 return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
             });
-        }
-
-        // ---------------- phase 3: column sums of e * w
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-            const floatx4 w4 = row_values(rr, i4, g);
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const floatx4 w4 = row_values(rr, i4, g_s);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+                for (int j = 0; j < 4; ++j) v16[4 * i4 + j] = w4[j];
+            }
+#pragma unroll 1
+            for (int t = 0; t < TPW; ++t) {
+                const floatx16 c = score_tile(t);
+                const bool real = (kbase + t * 32 + n_s) < a.Sk;
+                float sum = 0.f;
 #pragma unroll
-                for (int t = 0; t < TPW; ++t) col_acc[t] = fmaf(acc[t][4 * i4 + j], w4[j], col_acc[t]);
+                for (int i = 0; i < 16; ++i) sum = fmaf(real ? fast_exp2(fmaf(c[i], a.c, nm[i])) : 0.f, v16[i], sum);
+#pragma unroll
+                for (int u = 0; u < TPW; ++u)  // col_acc lives in registers: static index only
+                    if (u == t) col_acc[u] += sum;
             }
         }
     }
@@ -415,7 +447,7 @@ template <int TPW>
 static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.f_nqblk * p.B, p.f_hg);
-    if (p.Sk == p.f_kg * TPW * 32)
+    if (p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false>), grid, dim3(512), 0, st, a);
     else
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true>), grid, dim3(512), 0, st, a);
