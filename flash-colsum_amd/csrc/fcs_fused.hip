@@ -41,6 +41,10 @@ constexpr int kRedPitch = 40;             // floats per row of the wave-private 
 #define FCS_GLDS16(gptr, lptr)                                                                \
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gptr), \
                                      (__attribute__((address_space(3))) void *)(lptr), 16, 0, 0)
+// same, with an immediate byte offset that the hardware adds to BOTH the global and the LDS address
+#define FCS_GLDS16_OFF(gptr, lptr, OFF)                                                       \
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gptr), \
+                                     (__attribute__((address_space(3))) void *)(lptr), 16, OFF, 0)
 #define FCS_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
 // Hides a value's origin from the optimiser.  Used inside the walk over heads so that
 // per-tile addresses are formed where they are used instead of being precomputed for the
@@ -133,10 +137,11 @@ __device__ __forceinline__ floatx4 row_values(const RowRed &rr, int i4, int g)
 
 }  // namespace
 
-// RAGGED = false: S_k is exactly (key groups) x TPW x 32 and S_q a multiple of the block's rows:
-//                 every operand tile is whole, no padding keys anywhere.
-// RAGGED = true : tiles may run past the tensors; fetches clamp their rows and every exponent is
-//                 masked per lane.
+// RAGGED = false: S_k is exactly (key groups) x TPW x 32, S_q a multiple of the block's rows and
+//                 the rows of Q and K are dense (row stride == D): every operand tile is whole,
+//                 no padding keys anywhere, and tile addresses need no per-lane arithmetic.
+// RAGGED = true : anything else; fetches compute and clamp their rows per lane and every exponent
+//                 is masked per lane.
 template <int D, int TPW, bool RAGGED>
 __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 {
@@ -180,7 +185,8 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     uint32_t piece_b[2];   // byte offset in its row of the piece this lane fetches (even / odd instruction)
 #pragma unroll
     for (int par = 0; par < 2; ++par) piece_b[par] = (uint32_t)(((lane & 7) ^ ((par * 4 + (lane >> 4)) & 7)) * 16);
-    const uint32_t q_row_b = (uint32_t)a.qs_s * 2u, k_row_b = (uint32_t)a.ks_s * 2u;  // row pitch in bytes
+    // row pitch in bytes; a compile-time constant in the non-ragged kernel (rows are dense there)
+    const uint32_t q_row_b = RAGGED ? (uint32_t)a.qs_s * 2u : (uint32_t)(D * 2), k_row_b = RAGGED ? (uint32_t)a.ks_s * 2u : (uint32_t)(D * 2);
     uint32_t q_voff[2] = {lrow * q_row_b + piece_b[0], lrow * q_row_b + piece_b[1]};
     uint32_t k_voff[2] = {lrow * k_row_b + piece_b[0], lrow * k_row_b + piece_b[1]};
     const char *q_b = reinterpret_cast<const char *>(a.q + (int64_t)b * a.qs_b) + (int64_t)q0 * q_row_b;
@@ -194,16 +200,23 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // consumer masks or ignores them).  No branch either way: a taken branch costs a wave far
     // more than the few address instructions it would skip.
     auto fetch_piece = [&](const char *tile, uint32_t row_b, uint32_t (&voff)[2], int rows_left, int slot, int tt) {
-        char *dst = my_ring + slot * SLOT_BYTES + tt * 1024;
-        if (!RAGGED) {  // every tile is whole: scalar base + one 32-bit lane offset, no branch
+        char *dst = my_ring + slot * SLOT_BYTES;
+        if (!RAGGED) {
+            // every tile is whole and its rows are dense: instruction tt reads 1 KB further in
+            // memory and writes 1 KB further in the slot, which is exactly what the immediate
+            // offset does; base pointer, lane offset and LDS base are shared by the four pieces
+            static_assert(NT == 4, "offsets below");
             FCS_OPAQUE_V(voff[tt & 1]);
-            const char *rows8 = tile + (size_t)((uint32_t)(tt * 8) * row_b);
-            FCS_GLDS16(rows8 + voff[tt & 1], dst);
+            const char *src = tile + voff[tt & 1];
+            if (tt == 0) FCS_GLDS16_OFF(src, dst, 0);
+            else if (tt == 1) FCS_GLDS16_OFF(src, dst, 1024);
+            else if (tt == 2) FCS_GLDS16_OFF(src, dst, 2048);
+            else FCS_GLDS16_OFF(src, dst, 3072);
         } else {
             FCS_OPAQUE_V(lrow);
             FCS_OPAQUE_V(piece_b[tt & 1]);
             const uint32_t row = (uint32_t)max(0, min(tt * 8 + lrow, rows_left - 1));
-            FCS_GLDS16(tile + (row * row_b + piece_b[tt & 1]), dst);
+            FCS_GLDS16(tile + (row * row_b + piece_b[tt & 1]), dst + tt * 1024);
         }
     };
     // Read a ring slot back as an MFMA operand: lane (n, g) takes, for step tt, piece 2*tt + g of
@@ -447,7 +460,7 @@ template <int TPW>
 static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.f_nqblk * p.B, p.f_hg);
-    if (p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0)
+    if (p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false>), grid, dim3(512), 0, st, a);
     else
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true>), grid, dim3(512), 0, st, a);
