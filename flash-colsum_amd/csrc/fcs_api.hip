@@ -19,7 +19,7 @@ bool strides_ok(const int64_t s[4], bool use_batch)
     return true;
 }
 
-int run(int causal, const void *q, const void *k, float *out, void *ws, size_t ws_bytes, int B, int H,
+int run(int causal, const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes, int B, int H,
         int Sq, int Sk, int D, const int64_t qs[4], const int64_t ks[4], float scale, int cls_n,
         int k_past, void *stream)
 {
@@ -53,6 +53,7 @@ int run(int causal, const void *q, const void *k, float *out, void *ws, size_t w
     a.heads_per_group = p.heads_per_group; a.qtiles_per_group = p.qtiles_per_group;
     a.partial = reinterpret_cast<float *>(w + p.off_partial);
     a.out = out;
+    a.out_h = static_cast<_Float16 *>(out_f16);
     a.inv_norm = 1.0f / ((float)H * (float)p.q_rows);
     a.n_partials = p.n_partials;
     a.f_kg = p.f_kg; a.f_tpw = p.f_tpw; a.f_nqblk = p.f_nqblk; a.f_hpg = p.f_hpg;
@@ -87,19 +88,19 @@ size_t fcs_workspace_bytes(int causal, int B, int H, int Sq, int Sk, int D, int 
     return p.total;
 }
 
-int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *ws, size_t ws_bytes, int B, int H,
+int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes, int B, int H,
                              int S, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
                              int cls_n, void *hip_stream)
 {
-    return run(0, q, k, out, ws, ws_bytes, B, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
+    return run(0, q, k, out, out_f16, ws, ws_bytes, B, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
                hip_stream);
 }
 
-int fcs_colsum_causal_f16(const void *q, const void *k, float *out, void *ws, size_t ws_bytes, int H, int Q_len,
+int fcs_colsum_causal_f16(const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes, int H, int Q_len,
                           int K_len, int D, int k_past, const int64_t q_strides[4], const int64_t k_strides[4],
                           float scale, void *hip_stream)
 {
-    return run(1, q, k, out, ws, ws_bytes, 1, H, Q_len, K_len, D, q_strides, k_strides, scale, -1, k_past,
+    return run(1, q, k, out, out_f16, ws, ws_bytes, 1, H, Q_len, K_len, D, q_strides, k_strides, scale, -1, k_past,
                hip_stream);
 }
 

@@ -25,6 +25,7 @@ struct Args {
     int gh, gq, heads_per_group, qtiles_per_group;
     float *partial;  // [gh*gq][B][Sk]
     float *out;      // [B][Sk]
+    _Float16 *out_h; // [B][Sk] or nullptr: the same means rounded to fp16
     float inv_norm;  // 1 / (H * q_rows)
     int n_partials;  // slabs of `partial` that fcs_finalize_kernel adds up
     // fused single-kernel path (scores stay in registers)

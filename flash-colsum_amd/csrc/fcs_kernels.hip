@@ -327,9 +327,10 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
             v += __shfl_xor(v, 1);
             const int key = kw0 + na * 32 + acc_row(i, g);
             if (r == 0 && key < a.Sk) {
-                if (direct)
+                if (direct) {
                     a.out[(int64_t)b * a.Sk + key] = v * a.inv_norm;
-                else
+                    if (a.out_h) a.out_h[(int64_t)b * a.Sk + key] = (_Float16)(v * a.inv_norm);
+                } else
                     a.partial[((int64_t)grp * a.B + b) * a.Sk + key] = v;
             }
         }
@@ -346,6 +347,7 @@ __global__ __launch_bounds__(256) void fcs_finalize_kernel(const Args a)
     float s = 0.f;
     for (int gi = 0; gi < ng; ++gi) s += a.partial[(int64_t)gi * n + idx];
     a.out[idx] = s * a.inv_norm;
+    if (a.out_h) a.out_h[idx] = (_Float16)(s * a.inv_norm);
 }
 
 // ------------------------------------------------------------------------------------

@@ -16,7 +16,7 @@ from typing import Optional
 import torch
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libflashcolsum.so")
-_ABI_VERSION = 1
+_ABI_VERSION = 2
 _lib = None
 
 _I64x4 = ctypes.c_int64 * 4
@@ -40,13 +40,13 @@ def lib() -> ctypes.CDLL:
         cdll.fcs_workspace_bytes.argtypes = [ctypes.c_int] * 7
         cdll.fcs_colsum_noncausal_f16.restype = ctypes.c_int
         cdll.fcs_colsum_noncausal_f16.argtypes = [
-            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
             ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
             ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
             ctypes.c_float, ctypes.c_int, ctypes.c_void_p]
         cdll.fcs_colsum_causal_f16.restype = ctypes.c_int
         cdll.fcs_colsum_causal_f16.argtypes = [
-            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
             ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
             ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
             ctypes.c_float, ctypes.c_void_p]
@@ -84,7 +84,8 @@ def workspace_bytes(causal: bool, b: int, h: int, s_q: int, s_k: int, d: int, cl
     return int(lib().fcs_workspace_bytes(int(causal), b, h, s_q, s_k, d, cls_n))
 
 
-def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n: int, k_past: int) -> torch.Tensor:
+def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n: int, k_past: int, want_f16: bool = False):
+    """Enqueue one call; returns the fp32 means, or (fp32, fp16) when `want_f16`."""
     if q.device.type != "cuda" or k.device != q.device:
         raise ValueError(f"query and key must live on the same GPU, got {q.device} and {k.device}")
     q = _as_kernel_input(q)
@@ -93,20 +94,22 @@ def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n:
     s_k = k.shape[2]
     with torch.cuda.device(q.device):
         out = torch.empty((b, s_k), dtype=torch.float32, device=q.device)
+        out_h = torch.empty((b, s_k), dtype=torch.float16, device=q.device) if want_f16 else None
+        out_h_ptr = out_h.data_ptr() if want_f16 else None
         n_ws = workspace_bytes(causal, b, h, s_q, s_k, d, cls_n)
         ws = torch.empty((max(n_ws, 1),), dtype=torch.uint8, device=q.device)
         stream = torch.cuda.current_stream(q.device).cuda_stream
         qs, ks = _I64x4(*q.stride()), _I64x4(*k.stride())
         if causal:
             rc = lib().fcs_colsum_causal_f16(
-                q.data_ptr(), k.data_ptr(), out.data_ptr(), ws.data_ptr(), n_ws,
+                q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
                 h, s_q, s_k, d, int(k_past), qs, ks, float(scale), stream)
         else:
             rc = lib().fcs_colsum_noncausal_f16(
-                q.data_ptr(), k.data_ptr(), out.data_ptr(), ws.data_ptr(), n_ws,
+                q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
                 b, h, s_q, d, qs, ks, float(scale), int(cls_n), stream)
     _check(rc, "fcs_colsum_causal_f16" if causal else "fcs_colsum_noncausal_f16")
-    return out
+    return (out, out_h) if want_f16 else out
 
 
 def colsum_noncausal_f32(Q: torch.Tensor, K: torch.Tensor, scale: float, CLS_N: int = -1) -> torch.Tensor:
@@ -122,12 +125,17 @@ def colsum_causal_f32(Q: torch.Tensor, K: torch.Tensor, scale: float, K_past: Op
 
 
 def _flash_colsum_batched(Q, K, scale, CLS_N=-1):
-    return colsum_noncausal_f32(Q, K, scale, CLS_N).to(torch.float16)
+    """(B, S) fp16, like the reference launcher; the rounding happens in the final kernel."""
+    return _launch(False, Q, K, scale, -1 if CLS_N is None or CLS_N < 0 else int(CLS_N), 0, want_f16=True)[1]
 
 
 def _flash_colsum_non_batched(Q, K, scale, CLS_N=-1):
-    return colsum_noncausal_f32(Q, K, scale, CLS_N).to(torch.float16)
+    """(1, S) fp16; the same kernels serve B = 1 and B > 1."""
+    return _flash_colsum_batched(Q, K, scale, CLS_N)
 
 
 def _flash_colsum_causal(Q, K, scale, K_past=None):
-    return colsum_causal_f32(Q, K, scale, K_past).to(torch.float16)
+    """(1, K_len) fp16; K_past defaults to max(0, K_len - Q_len)."""
+    if K_past is None:
+        K_past = max(0, K.shape[2] - Q.shape[2])
+    return _launch(True, Q, K, scale, -1, int(K_past), want_f16=True)[1]

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FCS_ABI_VERSION 1
+#define FCS_ABI_VERSION 2
 
 enum {
     FCS_OK = 0,
@@ -56,13 +56,15 @@ size_t fcs_workspace_bytes(int causal, int B, int H, int Sq, int Sk, int D, int 
  *   q, k       (B,H,S,D) fp16, element strides q_strides[4] / k_strides[4] (HOST arrays);
  *              the last stride must be 1 and rows must be 16-byte aligned.
  *   out        (B,S) fp32 contiguous; receives the MEANS (already divided by H*rows).
+ *   out_f16    NULL, or (B,S) fp16 contiguous that additionally receives the means rounded
+ *              to fp16 (the reference's result dtype) without a separate cast kernel.
  *   cls_n      <= -1 (or any negative): average over all S query rows;
  *              >= 1: average over the first min(cls_n, S) query rows only.
  * Replaces `_flash_colsum_batched(Q, K, scale, CLS_N)` and
  * `_flash_colsum_non_batched(Q, K, scale, CLS_N)` including their host epilogue
  * (reference: flash_colsum/kernel_noncausal_batched.py:102-125,
  * flash_colsum/kernel_noncausal.py:95-117; called from flash_colsum/ops.py:102-105). */
-int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *ws, size_t ws_bytes,
+int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes,
                              int B, int H, int S, int D,
                              const int64_t q_strides[4], const int64_t k_strides[4],
                              float scale, int cls_n, void *hip_stream);
@@ -70,12 +72,13 @@ int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *ws,
 /* Causal column means for one sequence (batch 1), fp16 inputs, fp32 output.
  *   q          (1,H,Q_len,D), k (1,H,K_len,D) fp16; strides as above (index 0 ignored).
  *   out        (K_len) fp32; receives the means over the H*Q_len rows.
+ *   out_f16    NULL, or (K_len) fp16 that additionally receives the rounded means.
  *   k_past     number of keys every query may see before its own position: key j is
  *              visible to query i  <=>  j <= k_past + i.  The reference infers
  *              max(0, K_len - Q_len); pass that for drop-in behaviour.
  * Replaces `_flash_colsum_causal(Q, K, scale, K_past)` including its host epilogue
  * (reference: flash_colsum/kernel_causal.py:94-125; called from flash_colsum/ops.py:89). */
-int fcs_colsum_causal_f16(const void *q, const void *k, float *out, void *ws, size_t ws_bytes,
+int fcs_colsum_causal_f16(const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes,
                           int H, int Q_len, int K_len, int D, int k_past,
                           const int64_t q_strides[4], const int64_t k_strides[4],
                           float scale, void *hip_stream);

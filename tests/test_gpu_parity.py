@@ -66,17 +66,19 @@ def test_golden_vectors_through_c_abi(golden):
         n_ws = lib.fcs_workspace_bytes(int(c["causal"]), b, h, sq, sk, d, cls_n)
         ws = torch.empty(max(n_ws, 1), dtype=torch.uint8, device="cuda")
         out = torch.full((b, sk), float("nan"), dtype=torch.float32, device="cuda")
+        out_h = torch.full((b, sk), float("nan"), dtype=torch.float16, device="cuda")
         qs, ks = (ctypes.c_int64 * 4)(*q.stride()), (ctypes.c_int64 * 4)(*k.stride())
         stream = torch.cuda.current_stream().cuda_stream
         if c["causal"]:
-            rc = lib.fcs_colsum_causal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), ws.data_ptr(), n_ws, h, sq, sk,
-                                           d, max(0, sk - sq), qs, ks, scale, stream)
+            rc = lib.fcs_colsum_causal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h.data_ptr(), ws.data_ptr(),
+                                           n_ws, h, sq, sk, d, max(0, sk - sq), qs, ks, scale, stream)
         else:
-            rc = lib.fcs_colsum_noncausal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), ws.data_ptr(), n_ws, b, h,
-                                              sq, d, qs, ks, scale, cls_n, stream)
+            rc = lib.fcs_colsum_noncausal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h.data_ptr(), ws.data_ptr(),
+                                              n_ws, b, h, sq, d, qs, ks, scale, cls_n, stream)
         assert rc == 0, (name, _hip.strerror(rc))
         torch.cuda.synchronize()
         _assert_close(out, torch.from_numpy(c["out"]), name)
+        assert torch.equal(out_h, out.half()), name  # the fp16 output is the rounded fp32 output
 
 
 # ---------------------------------------------------------------------------------------

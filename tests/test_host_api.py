@@ -65,7 +65,7 @@ def test_library_exports_every_declared_symbol():
                      "fcs_workspace_bytes"]
     for n in names:
         assert getattr(lib, n) is not None
-    assert lib.fcs_abi_version() == 1
+    assert lib.fcs_abi_version() == 2
 
 
 def test_strerror_is_total():
@@ -93,20 +93,20 @@ def test_argument_errors_are_reported_without_a_gpu():
     unaligned = (ctypes.c_int64 * 4)(8 * 16 * 66, 16 * 66, 66, 1)
     p = ctypes.c_void_p(4096)  # never dereferenced: every call below fails its host checks
     nc, ca = lib.fcs_colsum_noncausal_f16, lib.fcs_colsum_causal_f16
-    assert nc(None, p, p, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
-    assert nc(p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
-    assert nc(p, p, p, p, 1 << 30, 0, 8, 16, 64, st, st, 0.125, -1, None) == -2
-    assert nc(p, p, p, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, 0, None) == -2
-    assert nc(p, p, p, p, 1 << 30, 2, 8, 16, 80, st, st, 0.125, -1, None) == -3
-    assert nc(p, p, p, p, 1 << 30, 2, 8, 16, 64, bad_last, st, 0.125, -1, None) == -4
-    assert nc(p, p, p, p, 1 << 30, 2, 8, 16, 64, st, unaligned, 0.125, -1, None) == -4
-    assert nc(ctypes.c_void_p(4098), p, p, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -4
-    assert nc(p, p, p, p, 16, 2, 8, 16, 64, st, st, 0.125, -1, None) == -5
-    assert nc(p, p, p, None, 0, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
-    assert nc(p, p, p, p, 1 << 30, 2, 8, 16, 64, st, st, float("nan"), -1, None) == -6
-    assert ca(p, p, p, p, 1 << 30, 8, 16, 64, 64, -1, st, st, 0.125, None) == -2
-    assert ca(p, p, p, p, 1 << 30, 8, 16, 64, 96, 48, st, st, 0.125, None) == -3
-    assert ca(p, p, p, p, 16, 8, 16, 64, 64, 48, st, st, 0.125, None) == -5
+    assert nc(None, p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
+    assert nc(p, p, None, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
+    assert nc(p, p, p, None, p, 1 << 30, 0, 8, 16, 64, st, st, 0.125, -1, None) == -2
+    assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, 0, None) == -2
+    assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 80, st, st, 0.125, -1, None) == -3
+    assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 64, bad_last, st, 0.125, -1, None) == -4
+    assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 64, st, unaligned, 0.125, -1, None) == -4
+    assert nc(ctypes.c_void_p(4098), p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -4
+    assert nc(p, p, p, None, p, 16, 2, 8, 16, 64, st, st, 0.125, -1, None) == -5
+    assert nc(p, p, p, None, None, 0, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
+    assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, float("nan"), -1, None) == -6
+    assert ca(p, p, p, None, p, 1 << 30, 8, 16, 64, 64, -1, st, st, 0.125, None) == -2
+    assert ca(p, p, p, None, p, 1 << 30, 8, 16, 64, 96, 48, st, st, 0.125, None) == -3
+    assert ca(p, p, p, None, p, 16, 8, 16, 64, 64, 48, st, st, 0.125, None) == -5
 
 
 def test_missing_library_is_loud(monkeypatch, tmp_path):
