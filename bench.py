@@ -38,7 +38,16 @@ WORKLOADS = {
     "causal_h32_q128_k16384_d128": ((1, 32, 128, 128), (1, 32, 16384, 128), dict(is_causal=True), False),
     "causal_h32_q512_k65536_d128_peaky": ((1, 32, 512, 128), (1, 32, 65536, 128), dict(is_causal=True), False),
 }
+KERNELS_OF = {
+    "noncausal_b2_h4_s512_d64": "fcs_fused_kernel<64,8,false> + fcs_finalize_kernel (one call)",
+    "noncausal_b8_h16_s2048_d64": "fcs_fused_kernel<64,8,false> + fcs_finalize_kernel (one call; the fused kernel is >= 96 % of it)",
+    "cls1_b32_h16_s577_d64": "fcs_fused_kernel<64,5,true> + fcs_finalize_kernel (one call)",
+    "causal_h32_q128_k4096_d128": "fcs_rowstats + fcs_merge_stats + fcs_colsum + fcs_finalize (one call)",
+    "causal_h32_q128_k16384_d128": "fcs_rowstats + fcs_merge_stats + fcs_colsum + fcs_finalize (one call)",
+    "causal_h32_q512_k65536_d128_peaky": "fcs_rowstats + fcs_merge_stats + fcs_colsum + fcs_finalize (one call)",
+}
 DEFAULT = "noncausal_b8_h16_s2048_d64"
+SETTLE_CALLS = 150  # untimed, before the --warmup steps
 
 
 def make_inputs(name):
@@ -74,6 +83,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy five times, so that a rocprofv3 --pmc run over this "
+                         "command sees a kernel of known HBM traffic next to the workload's kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this path has no multi-GPU part, run with --gpus 1")
@@ -89,7 +101,10 @@ def main():
     k = k32.half().cuda()
     torch.cuda.synchronize()
 
-    # ---- whole-call wall clock (the headline): K calls back to back between two syncs
+    # ---- whole-call wall clock (the headline): K calls back to back between two syncs.
+    # The GPU's clocks take a few tens of milliseconds of load to settle; untimed calls first.
+    for _ in range(SETTLE_CALLS):
+        flash_colsum(q, k, **kwargs)
     for _ in range(args.warmup):
         flash_colsum(q, k, **kwargs)
     torch.cuda.synchronize()
@@ -142,7 +157,7 @@ def main():
     ker_tflops = fl / (ker_ms * 1e-3) / 1e12
     roofline = {
         "bound": "mfma",
-        "kernel": "all kernels of one call (fcs_rowstats + fcs_colsum + fcs_finalize)",
+        "kernel": KERNELS_OF[name],
         "achieved": round(ker_tflops, 2),
         "peak": PEAK_FP16_TFLOPS,
         "unit": "TFLOP/s",
@@ -154,6 +169,19 @@ def main():
     }
     print(f"[bench] {name}: {ms_call:.4f} ms/call wall, {raw_ms:.4f} ms C-ABI back-to-back, {ker_ms:.4f} ms kernels, "
           f"{tflops:.1f} / {ker_tflops:.1f} TFLOP/s", file=sys.stderr)
+
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
+    # measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), bytes per call
+    traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file) as f:
+            roofline["traffic"] = json.load(f).get(name)
 
     # ---- CPU baseline: eager materialising path on the host cores, same workload
     cpu = None
@@ -180,8 +208,8 @@ def main():
         print(f"[bench] cpu baseline: {t_cpu * 1e3:.1f} ms/call on {torch.get_num_threads()} threads", file=sys.stderr)
 
     rec = {
-        "metric": "effective TFLOP/s (4*B*H*Sq*Sk*D per call, two QK^T passes) and ms/call, B8 H16 S2048 D64 non-causal"
-        if name == DEFAULT else f"effective TFLOP/s and ms/call, {name}",
+        "metric": "ms/call + effective TFLOP/s (% fp16 MFMA peak), B8 H16 S2048 D64 non-causal"
+        if name == DEFAULT else f"ms/call + effective TFLOP/s (% fp16 MFMA peak), {name}",
         "value": round(tflops, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -191,7 +219,8 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "fp16 MFMA inputs, fp32 accumulate/softmax",
+        "dtype": "fp16",
+        "dtype_note": "fp16 MFMA operands, fp32 accumulation, fp32 softmax and column sums",
         "data": "synthetic: N(0,1) from torch.Generator(seed 0) on CPU, rounded to fp16",
         "config": {"workload": name, "q_shape": list(q.shape), "k_shape": list(k.shape), **{k_: v for k_, v in kwargs.items()}},
         "frac_of_fp16_mfma_peak": round(tflops / PEAK_FP16_TFLOPS, 4),
