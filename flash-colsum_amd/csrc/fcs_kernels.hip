@@ -27,22 +27,25 @@ namespace fcs {
 // ------------------------------------------------------------------------------------
 // pass 1: per-row log-sum-exp (or per-split partials)
 // ------------------------------------------------------------------------------------
-template <int D, int QW>
-__global__ __launch_bounds__(256, 2) void fcs_rowstats_kernel(const Args a)
+// WAVES = 4 or 8 waves per block: a block covers WAVES * QW query rows and streams its keys
+// once, so taller blocks divide the key traffic of this pass.
+template <int D, int QW, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args a)
 {
+    constexpr int THREADS = 64 * WAVES;
     constexpr int NB = QW / 32;         // query fragments per wave
     constexpr int NT = D / 16;          // MFMA steps along the head dim
     constexpr int KT = kStageKeys;      // keys per LDS stage
     constexpr int NA = KT / 32;         // key fragments per stage
     constexpr int PITCH = D + 8;        // halves per LDS row (+16 B: conflict-free b128 reads)
     constexpr int CPR = D / 8;          // 16-byte pieces per row
-    constexpr int CPT = KT * CPR / 256; // pieces per thread per stage
+    constexpr int CPT = KT * CPR / THREADS;  // pieces per thread per stage
     __shared__ __attribute__((aligned(16))) _Float16 lds[2][KT * PITCH];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
     const int bh = blockIdx.z, b = bh / a.H, h = bh - b * a.H;
     const int chunk = blockIdx.y;
-    const int q0 = blockIdx.x * (4 * QW);
+    const int q0 = blockIdx.x * (WAVES * QW);
     const int qw0 = q0 + wave * QW;
     const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
     const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)h * a.ks_h;
@@ -50,7 +53,7 @@ __global__ __launch_bounds__(256, 2) void fcs_rowstats_kernel(const Args a)
     // key range of this block: its split, cut at the last key any of its rows may see
     const int kc0 = chunk * a.chunk_keys;
     int kc1 = min(a.Sk, kc0 + a.chunk_keys);
-    if (a.causal) kc1 = min(kc1, a.k_past + min(q0 + 4 * QW, a.q_rows));
+    if (a.causal) kc1 = min(kc1, a.k_past + min(q0 + WAVES * QW, a.q_rows));
     const int nst = (kc1 > kc0) ? (kc1 - kc0 + KT - 1) / KT : 0;
 
     half8 qf[NB][NT];
@@ -76,18 +79,112 @@ __global__ __launch_bounds__(256, 2) void fcs_rowstats_kernel(const Args a)
     auto gload = [&](int kb) {
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
-            const int c = tid + i * 256, row = c / CPR, col = (c % CPR) * 8;
+            const int c = tid + i * THREADS, row = c / CPR, col = (c % CPR) * 8;
             stg[i] = load8(kp + (int64_t)min(kb + row, a.Sk - 1) * a.ks_s + col);
         }
     };
     auto lstore = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
-            const int c = tid + i * 256, row = c / CPR, col = (c % CPR) * 8;
+            const int c = tid + i * THREADS, row = c / CPR, col = (c % CPR) * 8;
             *reinterpret_cast<half8 *>(&lds[buf][row * PITCH + col]) = stg[i];
         }
     };
 
+    // ---------------- common path: 2^(c*s) without max subtraction, exact while the row sums stay
+    // inside [2^-80, 2^120).  Software-pipelined over (key fragment x all query fragments) groups:
+    // the MFMAs of a group are issued before the exponent work of the previous group, so the
+    // matrix pipe and the VALU run together inside one wave.
+    bool redo;
+    {
+        float lacc[NB][4];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) lacc[nb][j] = 0.f;
+        floatx16 cp[NB];  // scores of the previous group, not yet exponentiated
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) cp[nb][i] = 0.f;
+        int p_kb = 0x3fffffff;  // key base of the previous group (the initial dummy hides every key)
+        auto drain = [&]() {
+            const bool edge = (p_kb + 31 > thr_min);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                if (!edge) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) lacc[nb][i & 3] += fast_exp2(cp[nb][i] * a.c);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const float e = fast_exp2(cp[nb][i] * a.c);
+                        lacc[nb][i & 3] += (p_kb + acc_row(i, g) <= thr[nb]) ? e : 0.f;
+                    }
+                }
+            }
+            // keeps the exponent work of this group between the MFMAs of the next two groups
+            if (NB == 2)
+                asm volatile("" : "+v"(lacc[0][0]), "+v"(lacc[0][1]), "+v"(lacc[0][2]), "+v"(lacc[0][3]), "+v"(lacc[NB - 1][0]),
+                             "+v"(lacc[NB - 1][1]), "+v"(lacc[NB - 1][2]), "+v"(lacc[NB - 1][3]));
+            else
+                asm volatile("" : "+v"(lacc[0][0]), "+v"(lacc[0][1]), "+v"(lacc[0][2]), "+v"(lacc[0][3]));
+        };
+
+        if (nst > 0) { gload(kc0); lstore(0); }
+        __syncthreads();
+        for (int it = 0; it < nst; ++it) {
+            const int kb = kc0 + it * KT;
+            if (it + 1 < nst) gload(kb + KT);
+            const _Float16 *tile = lds[it & 1];
+#pragma unroll
+            for (int na = 0; na < NA; ++na) {
+                half8 af[NT];
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    af[t] = *reinterpret_cast<const half8 *>(&tile[(na * 32 + r) * PITCH + t * 16 + g * 8]);
+                floatx16 cn[NB];
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) cn[nb][i] = 0.f;
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb)
+                        cn[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t], qf[nb][t], cn[nb], 0, 0, 0);
+                // the new MFMAs are in the instruction stream before the old scores are touched
+                if (NB == 2)
+                    asm volatile("" : "+v"(cn[0]), "+v"(cn[NB - 1]), "+v"(cp[0]), "+v"(cp[NB - 1]));
+                else
+                    asm volatile("" : "+v"(cn[0]), "+v"(cp[0]));
+                drain();
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) cp[nb] = cn[nb];
+                p_kb = kb + na * 32;
+            }
+            if (it + 1 < nst) lstore((it + 1) & 1);
+            __syncthreads();
+        }
+        drain();
+
+        bool bad = false;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const float lh = (lacc[nb][0] + lacc[nb][1]) + (lacc[nb][2] + lacc[nb][3]);
+            const float lt = lh + __shfl_xor(lh, 32);  // both half-waves: the chunk's full row sum
+            const bool has_keys = (nst > 0) && (kc0 <= thr[nb]);
+            bad = bad || (has_keys && !(lt >= 8.2718061e-25f && lt < 1.3292280e+36f));
+            m[nb] = has_keys ? 0.f : kNegBig;  // an empty split must not set the merged maximum
+            l[nb] = lh;
+        }
+        redo = __syncthreads_or(bad) != 0;
+    }
+
+    // ---------------- rare: online max-subtracted softmax over the same keys
+    if (redo) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) { m[nb] = kNegBig; l[nb] = 0.f; }
     if (nst > 0) { gload(kc0); lstore(0); }
     __syncthreads();
     for (int it = 0; it < nst; ++it) {
@@ -161,6 +258,8 @@ __global__ __launch_bounds__(256, 2) void fcs_rowstats_kernel(const Args a)
         __syncthreads();
     }
 
+    }  // redo
+
     // combine the two half-waves (same query, disjoint keys) and store
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
@@ -181,19 +280,29 @@ __global__ __launch_bounds__(256, 2) void fcs_rowstats_kernel(const Args a)
     }
 }
 
-// merge the per-split (max, sum) partials of pass 1 into lse2
-__global__ __launch_bounds__(256) void fcs_merge_stats_kernel(const Args a)
+// merge the per-split (max, sum) partials of pass 1 into lse2: one thread per row, eight partials
+// loaded at a time and folded in split order (fixed order: bit-reproducible)
+__global__ __launch_bounds__(64) void fcs_merge_stats_kernel(const Args a)
 {
-    const int i = blockIdx.x * 256 + threadIdx.x;
+    const int i = blockIdx.x * 64 + threadIdx.x;
     const int bh = blockIdx.y;
     if (i >= a.rows_pad) return;
     const float2 *p = a.ml + (int64_t)bh * a.n_chunks * a.rows_pad + i;
-    float mm = -INFINITY;
-    for (int c = 0; c < a.n_chunks; ++c) mm = fmaxf(mm, p[(int64_t)c * a.rows_pad].x);
-    float ll = 0.f;
-    for (int c = 0; c < a.n_chunks; ++c) {
-        const float2 v = p[(int64_t)c * a.rows_pad];
-        ll += v.y * fast_exp2(v.x - mm);
+    float mm = kNegBig * 4.f, ll = 0.f;
+    for (int c0 = 0; c0 < a.n_chunks; c0 += 8) {
+        float2 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            v[j].x = kNegBig * 4.f;
+            v[j].y = 0.f;
+            if (c0 + j < a.n_chunks) v[j] = p[(int64_t)(c0 + j) * a.rows_pad];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float mn = fmaxf(mm, v[j].x);
+            ll = ll * fast_exp2(mm - mn) + v[j].y * fast_exp2(v[j].x - mn);
+            mm = mn;
+        }
     }
     a.lse[(int64_t)bh * a.rows_pad + i] = mm + fast_log2(ll);
 }
@@ -239,8 +348,8 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
     half8 kf[NA][NT];
     half8 stg[CPT];
     float stg_lse = 0.f;
-    auto gload = [&](int s) {
-        const int h = h_begin + s / nt, t = t_begin + s % nt;
+    auto gload = [&](int hs_, int ti_) {  // head and query tile of the stage, counted from the group's first
+        const int h = h_begin + hs_, t = t_begin + ti_;
         const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
@@ -261,11 +370,12 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
         if (tid < QT) lse_s[buf][tid] = stg_lse;
     };
 
-    if (nst > 0) { gload(0); lstore(0); }
+    if (nst > 0) { gload(0, 0); lstore(0); }
     __syncthreads();
+    int hs = 0, ti = 0;  // head and query tile of stage s, advanced incrementally
     for (int s = 0; s < nst; ++s) {
-        const int hs = s / nt, t = t_begin + (s - hs * nt);
-        if (s - hs * nt == 0) {  // new head: fetch this wave's key fragments
+        const int t = t_begin + ti;
+        if (ti == 0) {  // new head: fetch this wave's key fragments
             const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)(h_begin + hs) * a.ks_h;
 #pragma unroll
             for (int na = 0; na < NA; ++na) {
@@ -277,7 +387,8 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
                 }
             }
         }
-        if (s + 1 < nst) gload(s + 1);
+        const int ti1 = (ti + 1 == nt) ? 0 : ti + 1, hs1 = (ti + 1 == nt) ? hs + 1 : hs;
+        if (s + 1 < nst) gload(hs1, ti1);
         const _Float16 *tile = lds[s & 1];
 
 #pragma unroll
@@ -288,21 +399,27 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
                 bf[tt] = *reinterpret_cast<const half8 *>(&tile[(nb * 32 + r) * PITCH + tt * 16 + g * 8]);
             const float nlse = -lse_s[s & 1][nb * 32 + r];
             const int qmin = t * QT + nb * 32;
-            const bool edge = a.causal && (kmax_w > a.k_past + qmin);  // wave-uniform
+            const bool edge = a.causal && (kmax_w > a.k_past + qmin);  // wave-uniform: straddles the diagonal
+            const int lim = a.k_past + qmin + r;                       // last key this lane's query sees
+            floatx16 cn[NA];
+#pragma unroll
+            for (int na = 0; na < NA; ++na)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) cn[na][i] = 0.f;
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt)
+#pragma unroll
+                for (int na = 0; na < NA; ++na)
+                    cn[na] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[na][tt], bf[tt], cn[na], 0, 0, 0);
 #pragma unroll
             for (int na = 0; na < NA; ++na) {
-                floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int tt = 0; tt < NT; ++tt)
-                    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[na][tt], bf[tt], c, 0, 0, 0);
                 if (!edge) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) colacc[na][i] += fast_exp2(fmaf(c[i], a.c, nlse));
+                    for (int i = 0; i < 16; ++i) colacc[na][i] += fast_exp2(fmaf(cn[na][i], a.c, nlse));
                 } else {
-                    const int lim = a.k_past + qmin + r;  // last key this lane's query sees
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
-                        const float p = fast_exp2(fmaf(c[i], a.c, nlse));
+                        const float p = fast_exp2(fmaf(cn[na][i], a.c, nlse));
                         colacc[na][i] += (kw0 + na * 32 + acc_row(i, g) <= lim) ? p : 0.f;
                     }
                 }
@@ -311,6 +428,8 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
 
         if (s + 1 < nst) lstore((s + 1) & 1);
         __syncthreads();
+        ti = ti1;
+        hs = hs1;
     }
 
     // sum the 32 query lanes of each half-wave; lane r == 0 of each half writes its 16 keys
@@ -377,16 +496,18 @@ static hipError_t launch_d(const Plan &p, const Args &a, hipStream_t st)
     const dim3 blk(256);
     {
         const dim3 grid(p.n_qblk, p.n_chunks, p.B * p.H);
-        if (p.qw == 64)
-            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64>), grid, blk, 0, st, a);
+        if (p.qw == 64 && p.k1_waves == 8)
+            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64, 8>), grid, dim3(512), 0, st, a);
+        else if (p.qw == 64)
+            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64, 4>), grid, blk, 0, st, a);
         else
-            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 32>), grid, blk, 0, st, a);
+            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 32, 4>), grid, blk, 0, st, a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     if (p.n_chunks > 1) {
-        const dim3 grid((p.rows_pad + 255) / 256, p.B * p.H);
-        hipLaunchKernelGGL(fcs_merge_stats_kernel, grid, blk, 0, st, a);
+        const dim3 grid((p.rows_pad + 63) / 64, p.B * p.H);
+        hipLaunchKernelGGL(fcs_merge_stats_kernel, grid, dim3(64), 0, st, a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

@@ -18,7 +18,8 @@ struct Plan {
     int q_rows;  // query rows that are averaged: min(cls_n, Sq) or Sq
     int causal, k_past;
     // pass 1: row statistics.  grid = (n_qblk, n_chunks, B*H)
-    int qw;          // query rows per wave (32 or 64); a block covers 4*qw rows
+    int qw;          // query rows per wave (32 or 64)
+    int k1_waves;    // waves per block (4 or 8); a block covers k1_waves*qw rows
     int n_qblk;      // blocks along the query axis
     int n_chunks;    // key-axis splits (partial (max,sum) per chunk when > 1)
     int chunk_keys;  // keys per split, multiple of kStageKeys
@@ -57,7 +58,8 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
 
     // ---- pass 1
     p.qw = (p.q_rows > 128) ? 64 : 32;
-    const int qblk = kWavesPerBlock * p.qw;
+    p.k1_waves = (p.q_rows > 256) ? 8 : 4;  // taller blocks re-read the keys less often
+    const int qblk = p.k1_waves * p.qw;
     p.n_qblk = ceil_div(p.q_rows, qblk);
     p.rows_pad = p.n_qblk * qblk;
     const long base1 = (long)p.n_qblk * B * H;
