@@ -142,10 +142,18 @@ __device__ __forceinline__ floatx4 row_values(const RowRed &rr, int i4, int g)
 //                 no padding keys anywhere, and tile addresses need no per-lane arithmetic.
 // RAGGED = true : anything else; fetches compute and clamp their rows per lane and every exponent
 //                 is masked per lane.
-template <int D, int TPW, bool RAGGED>
+// PRE = true (only with RAGGED = false, 8 key groups): the block's Q tile is multiplied by
+//                 c = scale * log2(e) in fp32 ONCE per head, rounded back to fp16 and shared by the
+//                 eight waves through LDS, so the scores leave the MFMAs already in the exponent's
+//                 unit and the per-score multiply disappears.  The extra fp16 rounding of Q perturbs
+//                 each score by ~2^-12 relative; the launcher only picks this variant when at least
+//                 4096 (head, row) pairs are averaged per output, where the effect on the means is
+//                 below 1e-4 relative (measured 6.5e-5 at B8 H16 S2048).
+template <int D, int TPW, bool RAGGED, bool PRE>
 __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 {
     static_assert(D == 64, "the fused path is laid out for 64-wide heads");
+    static_assert(!(PRE && RAGGED), "the pre-scaled variant needs whole tiles and dense rows");
     constexpr int NT = D / 16;             // MFMA steps (and 16-byte pieces per lane) per operand tile
     constexpr int NS = 3;                  // ring slots per wave
     constexpr int AHEAD = NS - 1;          // items in flight ahead of the one being consumed
@@ -156,6 +164,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     __shared__ __attribute__((aligned(16))) float red[8 * 32 * kRedPitch];
     __shared__ __attribute__((aligned(16))) float part[2 * 256];
     __shared__ __attribute__((aligned(16))) float wv[8 * 32];
+    __shared__ __attribute__((aligned(16))) char qshare[PRE ? 2 * 4096 : 16];  // pre-scaled Q tile, double-buffered
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what derives from it stays in SGPRs
@@ -265,11 +274,17 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     //     fetched into it; at most three items (12 DMA instructions) are in flight.
     //   * Past the last head the fetches repeat it, so that the number of outstanding DMA
     //     instructions at every wait is a compile-time constant.
+    // PRE: the Q item of a head is not a tile in the ring but this wave's 4 rows (512 B) of the raw
+    // tile, one ordinary 8-byte load per lane; the wave scales them and publishes them in `qshare`.
+    uint2 qraw = {0u, 0u};
+    auto item_vm = [&](int j_ahead) { return (PRE && (j_ahead % ITEMS) == 0) ? 1 : NT; };  // VMEM instructions of an item
     auto fetch_pos_piece = [&](int h_now, int j_ahead /* item index counted from the Q tile of head h_now, compile-time */,
                                int slot, int tt) {
         const int hh = min(h_now + j_ahead / ITEMS, h_end - 1);
         const int j = j_ahead % ITEMS;
-        if (j == 0)
+        if (j == 0 && PRE) {
+            if (tt == 0) qraw = *reinterpret_cast<const uint2 *>(q_b + (int64_t)hh * q_head_b + wave * 512 + lane * 8);
+        } else if (j == 0)
             fetch_piece(q_b + (int64_t)hh * q_head_b, q_row_b, q_voff, a.Sq - q0, slot, tt);
         else
             fetch_piece(k_b + (int64_t)hh * k_head_b + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff,
@@ -286,15 +301,45 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         return s_ >= NS ? s_ - NS : s_;
     };
 
+    // PRE: scale this wave's 4 raw rows by c (sign included) in fp32, round to fp16 and store them
+    // at their swizzled place in qshare[buf]; a workgroup barrier must follow before they are read
+    auto q_publish = [&](int buf) {
+        const float cs = a.negate ? -a.c : a.c;
+        const half8 raw = __builtin_bit_cast(half8, uint4v{qraw.x, qraw.y, 0u, 0u});
+        _Float16 sc[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sc[e] = (_Float16)((float)raw[e] * cs);
+        const int row = wave * 4 + (lane >> 4), pc = (lane & 15) >> 1, hf = lane & 1;
+        char *dst = qshare + buf * 4096 + row * 128 + ((pc ^ ((row >> 1) & 7)) * 16) + hf * 8;
+        *reinterpret_cast<uint2 *>(dst) = __builtin_bit_cast(uint2, *reinterpret_cast<const uint64_t *>(sc));
+    };
+    auto take_q_shared = [&](int buf, half8 (&dst)[NT]) {
+        const uint32_t diff = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)qshare + (uint32_t)(buf * 4096) -
+                              (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)my_ring;
+        const uint32_t ta0 = take_addr[0] + diff, ta1 = take_addr[1] + diff, ta2 = take_addr[2] + diff, ta3 = take_addr[3] + diff;
+        asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"
+                     : "=&v"(dst[0]), "=&v"(dst[1]), "=&v"(dst[2]), "=&v"(dst[3])
+                     : "v"(ta0), "v"(ta1), "v"(ta2), "v"(ta3)
+                     : "memory");
+    };
+
     half8 qf[NT], kf[2][NT];
 #pragma unroll
     for (int i = 0; i < NS; ++i) fetch_pos(h_begin, i, i);
+    if (PRE) {
+        q_publish(0);
+        __syncthreads();
+    }
 
     for (int unit = 0; unit < n_units; ++unit) {
         const int h = h_begin + unit;
         // this head's Q tile and first key tile (fetched during the previous head)
-        FCS_WAIT_VM(2 * NT);
-        take_issue(slot_of(0), qf);
+        if (PRE) {
+            take_q_shared(unit & 1, qf);
+        } else {
+            FCS_WAIT_VM(2 * NT);
+            take_issue(slot_of(0), qf);
+        }
         FCS_WAIT_VM(1 * NT);
         take_issue(slot_of(1), kf[0]);
         floatx16 acc[TPW];
@@ -307,7 +352,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             const bool real = !RAGGED || (kbase + t * 32 + n) < a.Sk;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const float e = real ? fast_exp2(acc[t][i] * a.c) : 0.f;
+                const float e = real ? fast_exp2(PRE ? acc[t][i] : acc[t][i] * a.c) : 0.f;
                 acc[t][i] = e;
                 rs[i] += e;
             }
@@ -325,7 +370,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             if (t == 0) {
                 take_wait(qf);
                 take_wait(kf[0]);
-                if (a.negate) {
+                if (!PRE && a.negate) {
 #pragma unroll
                     for (int tt = 0; tt < NT; ++tt) qf[tt] = flip_sign(qf[tt]);
                 }
@@ -335,7 +380,9 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 take_wait(kf[t & 1]);
                 fetch_pos(h, 1 + t + NS, slot_of(1 + t));
             }
-            FCS_WAIT_VM(2 * NT);  // the next key tile has landed; two later items may be in flight
+            // the next key tile has landed; the two items fetched after it may be in flight
+            if (item_vm(t + 3) + item_vm(t + 4) == 2 * NT) FCS_WAIT_VM(2 * NT);
+            else FCS_WAIT_VM(NT + 1);
             if (t + 1 < TPW) take_issue(slot_of(2 + t), kf[(t + 1) & 1]);
             floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -349,6 +396,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             sq += ITEMS % NS;
             if (sq >= NS) sq -= NS;
         }
+        if (PRE) q_publish((unit + 1) & 1);  // next head's Q tile; the reduction's barrier publishes it
 
         // ---------------- row sums over lanes and key-group waves; w = 1/L (0 for rows not averaged)
         const bool slow = reduce_rows<false>(rs, rr, kg_n, qg, kg, lane, [&](int row, float L) {
@@ -460,10 +508,13 @@ template <int TPW>
 static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.f_nqblk * p.B, p.f_hg);
-    if (p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64)
-        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false>), grid, dim3(512), 0, st, a);
+    const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
+    if (TPW == 8 && whole && p.f_kg == 8 && (long)p.H * p.q_rows >= 4096)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, (TPW == 8 ? 8 : 8), false, true>), grid, dim3(512), 0, st, a);
+    else if (whole)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false, false>), grid, dim3(512), 0, st, a);
     else
-        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true>), grid, dim3(512), 0, st, a);
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true, false>), grid, dim3(512), 0, st, a);
 }
 
 hipError_t launch_fused(const Plan &p, const Args &a, hipStream_t st)
