@@ -36,6 +36,7 @@ namespace {
 
 constexpr float kSumLo = 8.2718061e-25f;  // 2^-80
 constexpr float kSumHi = 1.3292280e+36f;  // 2^120
+constexpr float kSumHiPre = 268435456.f;  // 2^28: ceiling of the pre-scaled variant (bounds its score rounding error)
 constexpr int kRedPitch = 40;             // floats per row of the wave-private transpose buffer
 
 #define FCS_GLDS16(gptr, lptr)                                                                \
@@ -65,7 +66,8 @@ struct RowRed {
 // read back.  Returns (sum only) whether any row total of the WORKGROUP is outside
 // [2^-80, 2^120) or not finite; the answer is the same in every wave.  One barrier.
 template <bool MAX, typename Post>
-__device__ __forceinline__ bool reduce_rows(const float (&v)[16], RowRed &rr, int kg_n, int qg, int kg, int lane, Post post)
+__device__ __forceinline__ bool reduce_rows(const float (&v)[16], RowRed &rr, int kg_n, int qg, int kg, int lane, Post post,
+                                            const float sum_hi = kSumHi)
 {
     const int n = lane & 31, g = lane >> 5;
     // lanes: transpose through the wave's own LDS block (LDS executes a wave's accesses in order)
@@ -110,7 +112,7 @@ __device__ __forceinline__ bool reduce_rows(const float (&v)[16], RowRed &rr, in
     if (!MAX) {
         // every wave looks at all 256 partials of the workgroup: lane L at floats [4L, 4L + 4)
         const floatx4 f = reinterpret_cast<const floatx4 *>(part)[lane];
-        const bool hi = !(f[0] < kSumHi) || !(f[1] < kSumHi) || !(f[2] < kSumHi) || !(f[3] < kSumHi);
+        const bool hi = !(f[0] < sum_hi) || !(f[1] < sum_hi) || !(f[2] < sum_hi) || !(f[3] < sum_hi);
         const float m01 = fmaxf(f[0], f[1]), m23 = fmaxf(f[2], f[3]);
         float lowest;  // smallest per-row maximum over key groups among the rows this lane sees
         if (kg_n >= 4) {
@@ -401,7 +403,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         // ---------------- row sums over lanes and key-group waves; w = 1/L (0 for rows not averaged)
         const bool slow = reduce_rows<false>(rs, rr, kg_n, qg, kg, lane, [&](int row, float L) {
             return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
-        });
+        }, PRE ? kSumHiPre : kSumHi);
 
         if (!slow) {
             // ---------------- phase 3: column sums of e * w
@@ -509,7 +511,7 @@ static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.f_nqblk * p.B, p.f_hg);
     const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
-    if (TPW == 8 && whole && p.f_kg == 8 && (long)p.H * p.q_rows >= 4096)
+    if (TPW == 8 && whole && p.f_kg == 8 && (long)p.H * p.q_rows >= 4096 && fabsf(a.c) <= 0.1251f * 1.44269504f)
         hipLaunchKernelGGL((fcs_fused_kernel<64, (TPW == 8 ? 8 : 8), false, true>), grid, dim3(512), 0, st, a);
     else if (whole)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false, false>), grid, dim3(512), 0, st, a);

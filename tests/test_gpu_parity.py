@@ -219,6 +219,27 @@ def test_edge_shapes(qs, ks, kw):
     _assert_close(_run(q, k, **kw), _oracle(q, k, **kw), f"{qs} {ks} {kw}")
 
 
+@pytest.mark.parametrize("shape,same,kw,boost", [
+    ((1, 2, 2048, 64), False, {}, 0.0),                  # fewest averaged rows the variant accepts
+    ((1, 2, 2048, 64), True, {}, 0.0),                   # self-attention diagonal: largest scores
+    ((2, 4, 2048, 64), False, {"scale": -0.125}, 0.0),   # sign folded into the shared Q tile
+    ((1, 4, 2048, 64), False, {"scale": 0.1}, 0.0),
+    ((1, 4, 2048, 64), False, {"scale": 0.126}, 0.0),    # just above the variant's scale limit
+    ((1, 4, 2048, 64), False, {}, 6.0),                  # one head's scores exceed the variant's ceiling
+    ((1, 4, 2048, 64), True, {}, 40.0),                  # ... and the unstabilised range altogether
+])
+def test_prescaled_shared_q_variant(shape, same, kw, boost):
+    """Whole-tile S = 2048, D = 64 launches with >= 4096 averaged (head, row) pairs and
+    scale <= 1/8 run the fused kernel that scales Q once per head and rounds it to fp16;
+    heads whose row sums reach 2^28 must fall back to the exact path inside that kernel."""
+    q, k = _inputs(shape, shape, seed=11, same=same)
+    if boost:
+        q[:, 1, 100:164] *= boost
+        if same:
+            k = q.clone()
+    _assert_close(_run(q, k, **kw), _oracle(q, k, **kw), f"prescaled {shape} same={same} {kw} boost={boost}")
+
+
 def test_explicit_k_past():
     """The causal launcher's K_past argument (reference: kernel_causal.py:94-113)."""
     from flash_colsum import _hip
