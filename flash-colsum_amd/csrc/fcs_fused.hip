@@ -170,14 +170,16 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what derives from it stays in SGPRs
-    const int kg_n = a.f_kg, qg_n = 8 / kg_n;
+    const int kg_n = PRE ? 8 : a.f_kg, qg_n = 8 / kg_n;  // a constant folds the reduction's branches away
     const int qg = wave / kg_n, kg = wave - qg * kg_n;
     const int b = blockIdx.x % a.B, qblk = blockIdx.x / a.B;
     const int hgi = blockIdx.y;
     const int h_begin = hgi * a.f_hpg, h_end = min(a.H, h_begin + a.f_hpg);
     const int n_units = h_end - h_begin;
     const int blk_row0 = qblk * 32 * qg_n;  // first query row of the block
-    const int q0 = blk_row0 + qg * 32;      // first query row of this wave
+    // first query row of this wave; a wave whose rows all lie past the tensor re-reads the last row
+    // (its rows carry weight 0)
+    const int q0 = min(blk_row0 + qg * 32, a.Sq - 1);
     const int kbase = kg * TPW * 32;        // first key of this wave
 
     RowRed rr;

@@ -213,6 +213,10 @@ def test_reference_error_handling():
     ((2, 2, 64, 64), (2, 2, 64, 64), {"scale": 0.0}),
     ((1, 2, 90, 64), (1, 2, 400, 64), {"is_causal": True, "scale": 0.0}),
     ((2, 2, 200, 64), (2, 2, 200, 64), {"scale": 40.0}),
+    ((32, 1, 1000, 64), (32, 1, 1000, 64), {}),          # many batch entries, one head
+    ((36, 1, 950, 64), (36, 1, 950, 64), {}),            # ... with an odd number of query blocks
+    ((8, 2, 2048, 64), (8, 2, 2048, 64), {}),            # whole tiles, more workgroups than compute units
+    ((40, 2, 96, 64), (40, 2, 96, 64), {"cls_len": 5}),  # waves whose rows all lie past the tensor
 ])
 def test_edge_shapes(qs, ks, kw):
     q, k = _inputs(qs, ks, seed=3)
