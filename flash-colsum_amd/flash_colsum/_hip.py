@@ -80,8 +80,60 @@ def _as_kernel_input(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
+_ws_bytes_cache = {}
+
+
 def workspace_bytes(causal: bool, b: int, h: int, s_q: int, s_k: int, d: int, cls_n: int = -1) -> int:
-    return int(lib().fcs_workspace_bytes(int(causal), b, h, s_q, s_k, d, cls_n))
+    key = (bool(causal), b, h, s_q, s_k, d, cls_n)
+    n = _ws_bytes_cache.get(key)
+    if n is None:
+        n = int(lib().fcs_workspace_bytes(int(causal), b, h, s_q, s_k, d, cls_n))
+        if len(_ws_bytes_cache) < 4096:
+            _ws_bytes_cache[key] = n
+    return n
+
+
+# One workspace per (device, stream), grown on demand and reused by later calls: calls on one
+# stream execute in order, so the next call may overwrite what the previous one left behind.
+_workspaces = {}
+_WS_MIN_BYTES = 1 << 20
+
+
+def _workspace(device: torch.device, stream: int, n_bytes: int) -> torch.Tensor:
+    key = (device.index, stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < n_bytes:
+        ws = torch.empty((max(n_bytes, _WS_MIN_BYTES),), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def release_workspaces() -> None:
+    """Drop the cached per-stream workspaces (they are otherwise kept until the process ends)."""
+    _workspaces.clear()
+
+
+def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16):
+    b, h, s_q, d = q.shape
+    s_k = k.shape[2]
+    dev = q.device
+    out = torch.empty((b, s_k), dtype=torch.float32, device=dev)
+    out_h = torch.empty((b, s_k), dtype=torch.float16, device=dev) if want_f16 else None
+    out_h_ptr = out_h.data_ptr() if want_f16 else None
+    n_ws = workspace_bytes(causal, b, h, s_q, s_k, d, cls_n)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    ws = _workspace(dev, stream, n_ws)
+    qs, ks = _I64x4(*q.stride()), _I64x4(*k.stride())
+    if causal:
+        rc = lib().fcs_colsum_causal_f16(
+            q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
+            h, s_q, s_k, d, int(k_past), qs, ks, float(scale), stream)
+    else:
+        rc = lib().fcs_colsum_noncausal_f16(
+            q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
+            b, h, s_q, d, qs, ks, float(scale), int(cls_n), stream)
+    _check(rc, "fcs_colsum_causal_f16" if causal else "fcs_colsum_noncausal_f16")
+    return (out, out_h) if want_f16 else out
 
 
 def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n: int, k_past: int, want_f16: bool = False):
@@ -90,26 +142,10 @@ def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n:
         raise ValueError(f"query and key must live on the same GPU, got {q.device} and {k.device}")
     q = _as_kernel_input(q)
     k = _as_kernel_input(k)
-    b, h, s_q, d = q.shape
-    s_k = k.shape[2]
+    if q.device.index == torch.cuda.current_device():
+        return _enqueue(causal, q, k, scale, cls_n, k_past, want_f16)
     with torch.cuda.device(q.device):
-        out = torch.empty((b, s_k), dtype=torch.float32, device=q.device)
-        out_h = torch.empty((b, s_k), dtype=torch.float16, device=q.device) if want_f16 else None
-        out_h_ptr = out_h.data_ptr() if want_f16 else None
-        n_ws = workspace_bytes(causal, b, h, s_q, s_k, d, cls_n)
-        ws = torch.empty((max(n_ws, 1),), dtype=torch.uint8, device=q.device)
-        stream = torch.cuda.current_stream(q.device).cuda_stream
-        qs, ks = _I64x4(*q.stride()), _I64x4(*k.stride())
-        if causal:
-            rc = lib().fcs_colsum_causal_f16(
-                q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
-                h, s_q, s_k, d, int(k_past), qs, ks, float(scale), stream)
-        else:
-            rc = lib().fcs_colsum_noncausal_f16(
-                q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
-                b, h, s_q, d, qs, ks, float(scale), int(cls_n), stream)
-    _check(rc, "fcs_colsum_causal_f16" if causal else "fcs_colsum_noncausal_f16")
-    return (out, out_h) if want_f16 else out
+        return _enqueue(causal, q, k, scale, cls_n, k_past, want_f16)
 
 
 def colsum_noncausal_f32(Q: torch.Tensor, K: torch.Tensor, scale: float, CLS_N: int = -1) -> torch.Tensor:
