@@ -39,9 +39,9 @@ WORKLOADS = {
     "causal_h32_q512_k65536_d128_peaky": ((1, 32, 512, 128), (1, 32, 65536, 128), dict(is_causal=True), False),
 }
 KERNELS_OF = {
-    "noncausal_b2_h4_s512_d64": "fcs_fused_kernel<64,8,false> + fcs_finalize_kernel (one call)",
-    "noncausal_b8_h16_s2048_d64": "fcs_fused_kernel<64,8,false> + fcs_finalize_kernel (one call; the fused kernel is >= 96 % of it)",
-    "cls1_b32_h16_s577_d64": "fcs_fused_kernel<64,5,true> + fcs_finalize_kernel (one call)",
+    "noncausal_b2_h4_s512_d64": "fcs_fused_kernel<64,8,false,false> + fcs_finalize_kernel (one call)",
+    "noncausal_b8_h16_s2048_d64": "fcs_fused_kernel<64,8,false,true> + fcs_finalize_kernel (one call; the fused kernel is >= 96 % of it)",
+    "cls1_b32_h16_s577_d64": "fcs_fewrows_kernel<64,1> + fcs_finalize_kernel (one call)",
     "causal_h32_q128_k4096_d128": "fcs_rowstats + fcs_merge_stats + fcs_colsum + fcs_finalize (one call)",
     "causal_h32_q128_k16384_d128": "fcs_rowstats + fcs_merge_stats + fcs_colsum + fcs_finalize (one call)",
     "causal_h32_q512_k65536_d128_peaky": "fcs_rowstats + fcs_merge_stats + fcs_colsum + fcs_finalize (one call)",
@@ -71,9 +71,27 @@ def make_inputs(name):
 
 
 def flops(name):
+    """Nominal work of one call: two QK^T passes over all Sq rows, 4*B*H*Sq*Sk*D."""
     qs, ks, _, _ = WORKLOADS[name]
     b, h, sq, d = qs
     return 4.0 * b * h * sq * ks[2] * d
+
+
+def needed_rows(name):
+    qs, _, kwargs, _ = WORKLOADS[name]
+    return min(kwargs.get("cls_len") or qs[2], qs[2])
+
+
+def algorithmic_bytes(name):
+    """Bytes one call must move: the Q rows it averages, K, and the fp32 output."""
+    qs, ks, _, _ = WORKLOADS[name]
+    b, h, _, d = qs
+    return b * h * needed_rows(name) * d * 2 + ks[0] * ks[1] * ks[2] * d * 2 + ks[0] * ks[2] * 4
+
+
+def hbm_bound(name):
+    """With cls_len only a few query rows are needed: the call is a batch of GEMVs over K."""
+    return needed_rows(name) * 16 <= WORKLOADS[name][0][2] and needed_rows(name) <= 16
 
 
 def main():
@@ -155,6 +173,8 @@ def main():
     torch.cuda.synchronize()
     ker_ms = statistics.mean(e0.elapsed_time(e1) for e0, e1 in evs)
     ker_tflops = fl / (ker_ms * 1e-3) / 1e12
+    by = algorithmic_bytes(name)
+    ker_gbs = by / (ker_ms * 1e-3) / 1e9
     roofline = {
         "bound": "mfma",
         "kernel": KERNELS_OF[name],
@@ -165,8 +185,15 @@ def main():
         "kernel_ms": round(ker_ms, 5),
         "c_abi_back_to_back_ms": round(raw_ms, 5),
         "algorithmic_flops": fl,
+        "algorithmic_bytes": by,
+        "hbm_frac": round(ker_gbs / PEAK_HBM_GBS, 4),
         "traffic": None,
     }
+    if hbm_bound(name):
+        # only `cls_len` rows are needed, so the nominal FLOP count is not the work: price against HBM
+        roofline.update({"bound": "hbm", "achieved": round(ker_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(ker_gbs / PEAK_HBM_GBS, 4),
+                         "needed_tflops": round(fl * needed_rows(name) / q.shape[2] / (ker_ms * 1e-3) / 1e12, 3)})
     print(f"[bench] {name}: {ms_call:.4f} ms/call wall, {raw_ms:.4f} ms C-ABI back-to-back, {ker_ms:.4f} ms kernels, "
           f"{tflops:.1f} / {ker_tflops:.1f} TFLOP/s", file=sys.stderr)
 

@@ -40,6 +40,8 @@ int launch_colsum(const Plan &p, const Args &a, void *stream);
 
 // fused path, defined in fcs_fused.hip
 hipError_t launch_fused(const Plan &p, const Args &a, hipStream_t st);
+// few-rows path (fcs_fewrows.hip): p.fewrows == 1
+hipError_t launch_fewrows(const Plan &p, const Args &a, hipStream_t st);
 
 // shared final reduction out = inv_norm * sum of the n_partials slabs (fcs_kernels.hip)
 hipError_t launch_finalize(const Args &a, hipStream_t st);

@@ -530,6 +530,7 @@ static hipError_t launch_d(const Plan &p, const Args &a, hipStream_t st)
 int launch_colsum(const Plan &p, const Args &a, void *stream)
 {
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (p.fewrows) return (int)launch_fewrows(p, a, st);
     if (p.fused) return (int)launch_fused(p, a, st);
     hipError_t e = (p.D == 64) ? launch_d<64>(p, a, st) : launch_d<128>(p, a, st);
     return (int)e;

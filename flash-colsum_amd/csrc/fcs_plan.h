@@ -11,6 +11,8 @@ constexpr int kWavesPerBlock = 4;   // 256 threads
 constexpr int kStageKeys = 64;      // keys staged in LDS per step of the row-statistics pass
 constexpr int kStageRows = 64;      // query rows staged in LDS per step of the column pass
 constexpr int kFusedMaxKeys = 2048; // 8 waves x 8 tiles x 32 keys of fp32 scores per 32 query rows
+constexpr int kFewRowsMaxRows = 4;      // few-rows path: at most this many averaged query rows per head ...
+constexpr int kFewRowsMaxScores = 12288; // ... and rows * Sk scores (48 KB of LDS)
 constexpr int kTargetBlocks = 1024; // 256 CUs x 4: enough workgroups to fill the chip twice over
 
 struct Plan {
@@ -31,6 +33,7 @@ struct Plan {
     int heads_per_group, qtiles_per_group;
     // fused single-kernel path: non-causal, all keys of a row block fit in one
     // workgroup's registers.  grid = (f_nqblk * B, f_hg)
+    int fewrows;     // 1: few-rows path (non-causal, q_rows <= 4): grid = B * f_hg, slabs = f_hg
     int fused;       // 1: use it (then the two-pass fields above are unused)
     int f_kg, f_qg;  // waves along keys / along queries, f_kg * f_qg == 8
     int f_tpw;       // 32-key tiles per wave
@@ -87,8 +90,23 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     p.qtiles_per_group = ceil_div(n_qt, gq);
     p.gq = ceil_div(n_qt, p.qtiles_per_group);
 
-    // ---- fused path
+    // ---- few-rows path: a batch of matrix-vector products, one workgroup per (batch entry, head group)
+    p.fewrows = 0;
     p.fused = 0;
+    if (!causal && p.q_rows <= kFewRowsMaxRows && (long)p.q_rows * Sk <= kFewRowsMaxScores) {
+        p.fewrows = 1;
+        const long bh = (long)B * H;
+        int hpb = (int)((bh + 2047) / 2048);  // heads per workgroup: about 2048 workgroups at most
+        if (hpb > H) hpb = H;
+        p.f_hpg = hpb;
+        p.f_hg = ceil_div(H, hpb);
+        p.n_partials = p.f_hg;
+        p.off_lse = p.off_ml = p.off_partial = 0;
+        p.total = align256(sizeof(float) * (size_t)p.n_partials * B * Sk);
+        return true;
+    }
+
+    // ---- fused path
     p.n_partials = p.gh * p.gq;
     if (!causal && Sk <= kFusedMaxKeys && D == 64) {
         p.fused = 1;

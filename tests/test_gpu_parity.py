@@ -217,6 +217,17 @@ def test_reference_error_handling():
     ((36, 1, 950, 64), (36, 1, 950, 64), {}),            # ... with an odd number of query blocks
     ((8, 2, 2048, 64), (8, 2, 2048, 64), {}),            # whole tiles, more workgroups than compute units
     ((40, 2, 96, 64), (40, 2, 96, 64), {"cls_len": 5}),  # waves whose rows all lie past the tensor
+    # few averaged rows (matrix-vector path): every row count, both head dims, ragged key counts,
+    # several heads per workgroup, the largest score block it takes and the first it does not
+    ((3, 5, 577, 64), (3, 5, 577, 64), {"cls_len": 2}),
+    ((2, 3, 333, 128), (2, 3, 333, 128), {"cls_len": 4}),
+    ((2, 3, 7, 128), (2, 3, 7, 128), {"cls_len": 3}),
+    ((1, 2, 1, 64), (1, 2, 1, 64), {"cls_len": 1}),
+    ((300, 8, 64, 64), (300, 8, 64, 64), {"cls_len": 1}),
+    ((1, 4, 12288, 64), (1, 4, 12288, 64), {"cls_len": 1}),
+    ((1, 4, 5000, 64), (1, 4, 5000, 64), {"cls_len": 3}),
+    ((2, 4, 300, 64), (2, 4, 300, 64), {"cls_len": 2, "scale": -0.2}),
+    ((2, 4, 300, 128), (2, 4, 300, 128), {"cls_len": 1, "scale": 30.0}),
 ])
 def test_edge_shapes(qs, ks, kw):
     q, k = _inputs(qs, ks, seed=3)
