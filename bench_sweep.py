@@ -1,0 +1,123 @@
+#!/usr/bin/env python3
+"""Latency / peak-memory sweeps of `flash_colsum` on one MI355X, as CSV.
+
+Counterpart of the reference's three sweeps (reference: benchmarks/benchmark_colsum.py:289-424):
+
+  noncausal_batched   S = 1024, H = 16, D = 64, B in {1, 2, ..., 1024}
+  noncausal           B = 1, H = 16, D = 64, S in {2048, ..., 262144}
+  causal              B = 1, H = 32, Q_len = 128, D = 128, K_len in {16384, ..., 262144}
+
+Timing follows the reference's `measure_latency` (benchmark_colsum.py:42-56): warm-up calls,
+then `iters` x (call + device synchronize) under one wall clock, so launch and host overhead
+are included.  Peak memory is `torch.cuda.max_memory_allocated` around one call
+(benchmark_colsum.py:59-71); the kernels' workspace is allocated once per stream by the host
+layer and reported in its own column.  The eager baseline that materialises the attention matrix runs
+on the GPU too, and is skipped (empty CSV fields) when its score tensors would not fit.
+
+    python bench_sweep.py --sweep all --out sweep.csv
+"""
+import argparse
+import csv
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "flash-colsum_amd"))
+
+SWEEPS = {
+    "noncausal_batched": [dict(B=b, H=16, Sq=1024, Sk=1024, D=64, causal=False) for b in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024)],
+    "noncausal": [dict(B=1, H=16, Sq=s, Sk=s, D=64, causal=False) for s in (2048, 4096, 8192, 16384, 32768, 65536, 131072, 262144)],
+    "causal": [dict(B=1, H=32, Sq=128, Sk=k, D=128, causal=True) for k in (16384, 32768, 65536, 131072, 262144)],
+}
+EAGER_MAX_BYTES = 40 << 30  # logits + fp32 softmax + cast of the eager baseline must fit well inside HBM
+
+
+def measure_latency(fn, warmup, iters):
+    import torch
+
+    with torch.no_grad():
+        for _ in range(warmup):
+            fn()
+            torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+            torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / iters
+
+
+def peak_memory(fn):
+    import torch
+
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    with torch.no_grad():
+        fn()
+    torch.cuda.synchronize()
+    return torch.cuda.max_memory_allocated() - base
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--sweep", default="all", choices=sorted(SWEEPS) + ["all"])
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--out", default="-", help="CSV file, or - for stdout")
+    ap.add_argument("--no-eager", action="store_true", help="skip the eager baseline")
+    ap.add_argument("--max-points", type=int, default=0, help="only the first N points of each sweep (0 = all)")
+    args = ap.parse_args()
+
+    import torch
+    from flash_colsum import _hip, flash_colsum, naive_colsum
+
+    if not torch.cuda.is_available():
+        sys.exit("bench_sweep.py needs a GPU")
+    names = sorted(SWEEPS) if args.sweep == "all" else [args.sweep]
+    fields = ["sweep", "B", "H", "Sq", "Sk", "D", "causal", "flash_ms", "flash_peak_mib", "workspace_mib", "flash_tflops",
+              "eager_ms", "eager_peak_mib", "speedup", "max_abs_diff_vs_eager"]
+    out = sys.stdout if args.out == "-" else open(args.out, "w", newline="")
+    wr = csv.DictWriter(out, fieldnames=fields)
+    wr.writeheader()
+    for name in names:
+        points = SWEEPS[name][: args.max_points] if args.max_points else SWEEPS[name]
+        for pt in points:
+            g = torch.Generator(device="cuda").manual_seed(0)
+            q = torch.randn((pt["B"], pt["H"], pt["Sq"], pt["D"]), generator=g, device="cuda", dtype=torch.float16)
+            k = torch.randn((pt["B"], pt["H"], pt["Sk"], pt["D"]), generator=g, device="cuda", dtype=torch.float16)
+            scale = pt["D"] ** -0.5
+            run = lambda: flash_colsum(q, k, scale=scale, is_causal=pt["causal"])
+            # long points: fewer iterations, at least 3
+            t_probe = measure_latency(run, 1, 1)
+            iters = max(3, min(args.iters, int(2.0 / max(t_probe, 1e-6))))
+            t_fast = measure_latency(run, min(args.warmup, iters), iters)
+            m_fast = peak_memory(run)
+            row = dict(sweep=name, causal=int(pt["causal"]), flash_ms=round(t_fast * 1e3, 4),
+                       flash_peak_mib=round(m_fast / 2**20, 2),
+                       # kept by the host layer between calls, so not part of the per-call peak
+                       workspace_mib=round(_hip.workspace_bytes(pt["causal"], pt["B"], pt["H"], pt["Sq"], pt["Sk"], pt["D"]) / 2**20, 2),
+                       flash_tflops=round(4.0 * pt["B"] * pt["H"] * pt["Sq"] * pt["Sk"] * pt["D"] / t_fast / 1e12, 1),
+                       **{f: pt[f] for f in ("B", "H", "Sq", "Sk", "D")})
+            scores = pt["B"] * pt["H"] * pt["Sq"] * pt["Sk"]
+            if not args.no_eager and scores * (2 + 4 + 2 + 2) <= EAGER_MAX_BYTES:
+                ref = lambda: naive_colsum(q, k, scale=scale, is_causal=pt["causal"])
+                try:
+                    t_ref = measure_latency(ref, 1, max(3, min(iters, int(1.0 / max(t_fast * 20, 1e-6)) or 3)))
+                    m_ref = peak_memory(ref)
+                    diff = (run().float() - ref().float()).abs().max().item()
+                    row.update(eager_ms=round(t_ref * 1e3, 4), eager_peak_mib=round(m_ref / 2**20, 2),
+                               speedup=round(t_ref / t_fast, 2), max_abs_diff_vs_eager=f"{diff:.3e}")
+                except torch.OutOfMemoryError:
+                    torch.cuda.empty_cache()
+            wr.writerow(row)
+            out.flush()
+            print(f"[sweep] {name} {pt}: {row['flash_ms']} ms, eager {row.get('eager_ms')}", file=sys.stderr, flush=True)
+            del q, k
+            torch.cuda.empty_cache()
+    if out is not sys.stdout:
+        out.close()
+
+
+if __name__ == "__main__":
+    main()

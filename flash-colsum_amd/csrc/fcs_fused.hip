@@ -172,8 +172,20 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what derives from it stays in SGPRs
     const int kg_n = PRE ? 8 : a.f_kg, qg_n = 8 / kg_n;  // a constant folds the reduction's branches away
     const int qg = wave / kg_n, kg = wave - qg * kg_n;
-    const int b = blockIdx.x % a.B, qblk = blockIdx.x / a.B;
-    const int hgi = blockIdx.y;
+    // Workgroups are handed to the 8 XCDs round-robin in launch order, and each XCD has its own L2.
+    // The row blocks of one (head group, batch entry) read the same K, so they should run on one
+    // XCD and close together in time: XCD x, which receives workgroups x, x + 8, x + 16, ..., walks
+    // a contiguous range of the (head group, batch entry, row block) list, row blocks fastest.
+    int hgi, b, qblk;
+    {
+        const int n_all = gridDim.x * gridDim.y, i = blockIdx.y * gridDim.x + blockIdx.x;
+        const int x = i & 7, per = n_all >> 3, rem = n_all & 7;  // XCD x holds per + (x < rem) workgroups
+        const int v = x * per + min(x, rem) + (i >> 3);
+        qblk = v % a.f_nqblk;
+        const int t = v / a.f_nqblk;
+        b = t % a.B;
+        hgi = t / a.B;
+    }
     const int h_begin = hgi * a.f_hpg, h_end = min(a.H, h_begin + a.f_hpg);
     const int n_units = h_end - h_begin;
     const int blk_row0 = qblk * 32 * qg_n;  // first query row of the block
