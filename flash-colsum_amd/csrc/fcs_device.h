@@ -40,4 +40,22 @@ static constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
 static constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7 - i within groups of 8
 static constexpr int kDppMirror = 0x140;      // lane i <-> 15 - i within rows of 16
 
+// Workgroups are handed to the 8 XCDs round-robin in launch order (x fastest, then y, then z), and
+// each XCD has its own L2.  Neighbours along x usually read the same operand, so they should
+// run on one XCD and close together in time.  This returns the grid coordinates a workgroup should
+// work on instead of its own: XCD c, which receives workgroups c, c + 8, c + 16, ..., then walks a
+// contiguous range of the x-fastest list of all coordinates.  A bijection for any grid size.
+__device__ __forceinline__ void xcd_contiguous_block(int &bx, int &by, int &bz)
+{
+    const int nx = gridDim.x, ny = gridDim.y;
+    const int n_all = nx * ny * (int)gridDim.z;
+    const int i = ((int)blockIdx.z * ny + (int)blockIdx.y) * nx + (int)blockIdx.x;
+    const int c = i & 7, per = n_all >> 3, rem = n_all & 7;  // XCD c holds per + (c < rem) workgroups
+    const int v = c * per + min(c, rem) + (i >> 3);
+    bx = v % nx;
+    const int t = v / nx;
+    by = t % ny;
+    bz = t / ny;
+}
+
 }  // namespace fcs

@@ -172,19 +172,15 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what derives from it stays in SGPRs
     const int kg_n = PRE ? 8 : a.f_kg, qg_n = 8 / kg_n;  // a constant folds the reduction's branches away
     const int qg = wave / kg_n, kg = wave - qg * kg_n;
-    // Workgroups are handed to the 8 XCDs round-robin in launch order, and each XCD has its own L2.
-    // The row blocks of one (head group, batch entry) read the same K, so they should run on one
-    // XCD and close together in time: XCD x, which receives workgroups x, x + 8, x + 16, ..., walks
-    // a contiguous range of the (head group, batch entry, row block) list, row blocks fastest.
+    // The row blocks of one (head group, batch entry) read the same K: they run on one XCD, close
+    // together in time.
     int hgi, b, qblk;
     {
-        const int n_all = gridDim.x * gridDim.y, i = blockIdx.y * gridDim.x + blockIdx.x;
-        const int x = i & 7, per = n_all >> 3, rem = n_all & 7;  // XCD x holds per + (x < rem) workgroups
-        const int v = x * per + min(x, rem) + (i >> 3);
-        qblk = v % a.f_nqblk;
-        const int t = v / a.f_nqblk;
-        b = t % a.B;
-        hgi = t / a.B;
+        int bx, by, bz;
+        xcd_contiguous_block(bx, by, bz);
+        qblk = bx % a.f_nqblk;
+        b = bx / a.f_nqblk;
+        hgi = by;
     }
     const int h_begin = hgi * a.f_hpg, h_end = min(a.H, h_begin + a.f_hpg);
     const int n_units = h_end - h_begin;
@@ -523,7 +519,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 template <int TPW>
 static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
-    const dim3 grid(p.f_nqblk * p.B, p.f_hg);
+    const dim3 grid(p.f_nqblk * p.B, p.f_hg);  // x = batch entry * f_nqblk + row block
     const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
     if (TPW == 8 && whole && p.f_kg == 8 && (long)p.H * p.q_rows >= 4096 && fabsf(a.c) <= 0.1251f * 1.44269504f)
         hipLaunchKernelGGL((fcs_fused_kernel<64, (TPW == 8 ? 8 : 8), false, true>), grid, dim3(512), 0, st, a);

@@ -43,9 +43,11 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
     __shared__ __attribute__((aligned(16))) _Float16 lds[2][KT * PITCH];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
-    const int bh = blockIdx.z, b = bh / a.H, h = bh - b * a.H;
-    const int chunk = blockIdx.y;
-    const int q0 = blockIdx.x * (WAVES * QW);
+    int bx, by, bz;  // row blocks of one (key split, head) read the same keys: same XCD
+    xcd_contiguous_block(bx, by, bz);
+    const int bh = bz, b = bh / a.H, h = bh - b * a.H;
+    const int chunk = by;
+    const int q0 = bx * (WAVES * QW);
     const int qw0 = q0 + wave * QW;
     const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
     const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)h * a.ks_h;
@@ -324,9 +326,11 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
     __shared__ float lse_s[2][QT];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
-    const int b = blockIdx.z;
-    const int grp = blockIdx.y, gh_i = grp / a.gq, gq_i = grp - gh_i * a.gq;
-    const int k0 = blockIdx.x * (4 * KW);
+    int bx, by, bz;  // key blocks of one (group, batch entry) stream the same query tiles: same XCD
+    xcd_contiguous_block(bx, by, bz);
+    const int b = bz;
+    const int grp = by, gh_i = grp / a.gq, gq_i = grp - gh_i * a.gq;
+    const int k0 = bx * (4 * KW);
     const int kw0 = k0 + wave * KW;
     const int kmax_w = kw0 + KW - 1;
 
