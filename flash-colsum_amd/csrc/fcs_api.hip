@@ -19,7 +19,7 @@ bool strides_ok(const int64_t s[4], bool use_batch)
     return true;
 }
 
-int run(int causal, const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes, int B, int H,
+int run(int bf16, int causal, const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes, int B, int H,
         int Sq, int Sk, int D, const int64_t qs[4], const int64_t ks[4], float scale, int cls_n,
         int k_past, void *stream)
 {
@@ -32,6 +32,7 @@ int run(int causal, const void *q, const void *k, float *out, void *out_f16, voi
 
     fcs::Plan p;
     if (!fcs::make_plan(p, causal, B, H, Sq, Sk, D, cls_n, k_past)) return FCS_E_DIMS;
+    p.bf16 = bf16;
     if (p.total > 0 && (!ws || ws_bytes < p.total)) return ws ? FCS_E_WORKSPACE : FCS_E_NULL;
 
     fcs::Args a;
@@ -92,7 +93,15 @@ int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *out
                              int S, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
                              int cls_n, void *hip_stream)
 {
-    return run(0, q, k, out, out_f16, ws, ws_bytes, B, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
+    return run(0, 0, q, k, out, out_f16, ws, ws_bytes, B, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
+               hip_stream);
+}
+
+int fcs_colsum_noncausal_bf16(const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes, int B, int H,
+                              int S, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
+                              int cls_n, void *hip_stream)
+{
+    return run(1, 0, q, k, out, out_f16, ws, ws_bytes, B, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
                hip_stream);
 }
 
@@ -100,7 +109,15 @@ int fcs_colsum_causal_f16(const void *q, const void *k, float *out, void *out_f1
                           int K_len, int D, int k_past, const int64_t q_strides[4], const int64_t k_strides[4],
                           float scale, void *hip_stream)
 {
-    return run(1, q, k, out, out_f16, ws, ws_bytes, 1, H, Q_len, K_len, D, q_strides, k_strides, scale, -1, k_past,
+    return run(0, 1, q, k, out, out_f16, ws, ws_bytes, 1, H, Q_len, K_len, D, q_strides, k_strides, scale, -1, k_past,
+               hip_stream);
+}
+
+int fcs_colsum_causal_bf16(const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes, int H, int Q_len,
+                           int K_len, int D, int k_past, const int64_t q_strides[4], const int64_t k_strides[4],
+                           float scale, void *hip_stream)
+{
+    return run(1, 1, q, k, out, out_f16, ws, ws_bytes, 1, H, Q_len, K_len, D, q_strides, k_strides, scale, -1, k_past,
                hip_stream);
 }
 

@@ -9,6 +9,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 static constexpr float kNegBig = -1.0e30f;  // "hidden" score: finite so that max/sub never make NaN
 
@@ -22,6 +23,18 @@ __device__ __forceinline__ half8 flip_sign(half8 v)
     uint4v u = __builtin_bit_cast(uint4v, v);
     u ^= 0x80008000u;
     return __builtin_bit_cast(half8, u);
+}
+
+// One 32x32x16 MFMA step, fp32 accumulate.  The operands are 8 fp16 or (BF) 8 bf16 values per
+// lane; both travel through the kernels as the same 16-byte bit pattern (`half8`), and the sign
+// flip above works for either because the sign bits sit in the same places.
+template <bool BF>
+__device__ __forceinline__ floatx16 mfma16(half8 a, half8 b, floatx16 c)
+{
+    if constexpr (BF)
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 }
 
 // Row of a 32x32 MFMA result tile held by accumulator register i of a lane in half-wave g

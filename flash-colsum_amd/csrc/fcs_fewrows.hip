@@ -32,13 +32,24 @@ __device__ __forceinline__ float row_lanes_sum(float v)
     return v;
 }
 
+// dot product of 8 fp16 or (BF) 8 bf16 values per operand, fp32 accumulate
+template <bool BF>
 __device__ __forceinline__ float dot8(half8 x, half8 y)
 {
     float s = 0.f;
+    if constexpr (BF) {
+        const uint4v xu = __builtin_bit_cast(uint4v, x), yu = __builtin_bit_cast(uint4v, y);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const half2v xa = {x[2 * i], x[2 * i + 1]}, ya = {y[2 * i], y[2 * i + 1]};
-        s = __builtin_amdgcn_fdot2(xa, ya, s, false);
+        for (int i = 0; i < 4; ++i) {  // a bf16 value is the upper half of the fp32 with the same value
+            s = fmaf(__builtin_bit_cast(float, xu[i] << 16), __builtin_bit_cast(float, yu[i] << 16), s);
+            s = fmaf(__builtin_bit_cast(float, xu[i] & 0xffff0000u), __builtin_bit_cast(float, yu[i] & 0xffff0000u), s);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const half2v xa = {x[2 * i], x[2 * i + 1]}, ya = {y[2 * i], y[2 * i + 1]};
+            s = __builtin_amdgcn_fdot2(xa, ya, s, false);
+        }
     }
     return s;
 }
@@ -60,7 +71,7 @@ __device__ __forceinline__ float block_reduce(float v, float *slot, int lane, in
     return MAX ? fmaxf(fmaxf(a0, a1), fmaxf(a2, a3)) : (a0 + a1) + (a2 + a3);
 }
 
-template <int D, int R>
+template <int D, int R, bool BF>
 __global__ __launch_bounds__(256) void fcs_fewrows_kernel(const Args a)
 {
     constexpr int LPR = D / 8;     // lanes per key row (16 bytes each)
@@ -98,7 +109,7 @@ __global__ __launch_bounds__(256) void fcs_fewrows_kernel(const Args a)
                 const int row = base + u * RPB + wave * RPW + rw;
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    const float s = row_lanes_sum<LPR>(dot8(qv[r], kv[u]));
+                    const float s = row_lanes_sum<LPR>(dot8<BF>(qv[r], kv[u]));
                     if (sub == 0 && row < Sk) sc[r * Sk + row] = s * a.c;
                 }
             }
@@ -130,15 +141,15 @@ __global__ __launch_bounds__(256) void fcs_fewrows_kernel(const Args a)
     }
 }
 
-template <int D>
+template <int D, bool BF>
 static hipError_t launch_fewrows_d(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.B * p.f_hg), block(256);
     switch (p.q_rows) {
-    case 1: hipLaunchKernelGGL((fcs_fewrows_kernel<D, 1>), grid, block, 0, st, a); break;
-    case 2: hipLaunchKernelGGL((fcs_fewrows_kernel<D, 2>), grid, block, 0, st, a); break;
-    case 3: hipLaunchKernelGGL((fcs_fewrows_kernel<D, 3>), grid, block, 0, st, a); break;
-    case 4: hipLaunchKernelGGL((fcs_fewrows_kernel<D, 4>), grid, block, 0, st, a); break;
+    case 1: hipLaunchKernelGGL((fcs_fewrows_kernel<D, 1, BF>), grid, block, 0, st, a); break;
+    case 2: hipLaunchKernelGGL((fcs_fewrows_kernel<D, 2, BF>), grid, block, 0, st, a); break;
+    case 3: hipLaunchKernelGGL((fcs_fewrows_kernel<D, 3, BF>), grid, block, 0, st, a); break;
+    case 4: hipLaunchKernelGGL((fcs_fewrows_kernel<D, 4, BF>), grid, block, 0, st, a); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -146,7 +157,11 @@ static hipError_t launch_fewrows_d(const Plan &p, const Args &a, hipStream_t st)
 
 hipError_t launch_fewrows(const Plan &p, const Args &a, hipStream_t st)
 {
-    const hipError_t e = (p.D == 64) ? launch_fewrows_d<64>(p, a, st) : launch_fewrows_d<128>(p, a, st);
+    hipError_t e;
+    if (p.bf16)
+        e = (p.D == 64) ? launch_fewrows_d<64, true>(p, a, st) : launch_fewrows_d<128, true>(p, a, st);
+    else
+        e = (p.D == 64) ? launch_fewrows_d<64, false>(p, a, st) : launch_fewrows_d<128, false>(p, a, st);
     if (e != hipSuccess) return e;
     return launch_finalize(a, st);
 }

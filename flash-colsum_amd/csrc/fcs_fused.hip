@@ -151,11 +151,12 @@ __device__ __forceinline__ floatx4 row_values(const RowRed &rr, int i4, int g)
 //                 each score by ~2^-12 relative; the launcher only picks this variant when at least
 //                 4096 (head, row) pairs are averaged per output, where the effect on the means is
 //                 below 1e-4 relative (measured 6.5e-5 at B8 H16 S2048).
-template <int D, int TPW, bool RAGGED, bool PRE>
+template <int D, int TPW, bool RAGGED, bool PRE, bool BF>
 __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 {
     static_assert(D == 64, "the fused path is laid out for 64-wide heads");
     static_assert(!(PRE && RAGGED), "the pre-scaled variant needs whole tiles and dense rows");
+    static_assert(!(PRE && BF), "the pre-scaled variant rounds Q*c to fp16; bf16 would be too coarse");
     constexpr int NT = D / 16;             // MFMA steps (and 16-byte pieces per lane) per operand tile
     constexpr int NS = 3;                  // ring slots per wave
     constexpr int AHEAD = NS - 1;          // items in flight ahead of the one being consumed
@@ -398,7 +399,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             if (t + 1 < TPW) take_issue(slot_of(2 + t), kf[(t + 1) & 1]);
             floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int tt = 0; tt < NT; ++tt) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[tt], kf[t & 1][tt], c, 0, 0, 0);
+            for (int tt = 0; tt < NT; ++tt) c = mfma16<BF>(qf[tt], kf[t & 1][tt], c);
             acc[t] = c;
             if (t > 0) exp_tile(t - 1);  // VALU work of the previous tile runs under this tile's MFMAs
         }
@@ -451,7 +452,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 for (int tt = 0; tt < NT; ++tt) ks[tt] = load8(kp + (int64_t)krow * a.ks_s + tt * 16);
                 floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int tt = 0; tt < NT; ++tt) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(qs[tt], ks[tt], c, 0, 0, 0);
+                for (int tt = 0; tt < NT; ++tt) c = mfma16<BF>(qs[tt], ks[tt], c);
                 return c;
             };
             float v16[16];
@@ -516,32 +517,39 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     }
 }
 
-template <int TPW>
+template <int TPW, bool BF>
 static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.f_nqblk * p.B, p.f_hg);  // x = batch entry * f_nqblk + row block
     const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
-    if (TPW == 8 && whole && p.f_kg == 8 && (long)p.H * p.q_rows >= 4096 && fabsf(a.c) <= 0.1251f * 1.44269504f)
-        hipLaunchKernelGGL((fcs_fused_kernel<64, (TPW == 8 ? 8 : 8), false, true>), grid, dim3(512), 0, st, a);
+    if (!BF && TPW == 8 && whole && p.f_kg == 8 && (long)p.H * p.q_rows >= 4096 && fabsf(a.c) <= 0.1251f * 1.44269504f)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, true, false>), grid, dim3(512), 0, st, a);
     else if (whole)
-        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false, false>), grid, dim3(512), 0, st, a);
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false, false, BF>), grid, dim3(512), 0, st, a);
     else
-        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true, false>), grid, dim3(512), 0, st, a);
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true, false, BF>), grid, dim3(512), 0, st, a);
+}
+
+template <bool BF>
+static bool launch_fused_t(const Plan &p, const Args &a, hipStream_t st)
+{
+    switch (p.f_tpw) {
+    case 1: launch_tpw<1, BF>(p, a, st); break;
+    case 2: launch_tpw<2, BF>(p, a, st); break;
+    case 3: launch_tpw<3, BF>(p, a, st); break;
+    case 4: launch_tpw<4, BF>(p, a, st); break;
+    case 5: launch_tpw<5, BF>(p, a, st); break;
+    case 6: launch_tpw<6, BF>(p, a, st); break;
+    case 7: launch_tpw<7, BF>(p, a, st); break;
+    case 8: launch_tpw<8, BF>(p, a, st); break;
+    default: return false;
+    }
+    return true;
 }
 
 hipError_t launch_fused(const Plan &p, const Args &a, hipStream_t st)
 {
-    switch (p.f_tpw) {
-    case 1: launch_tpw<1>(p, a, st); break;
-    case 2: launch_tpw<2>(p, a, st); break;
-    case 3: launch_tpw<3>(p, a, st); break;
-    case 4: launch_tpw<4>(p, a, st); break;
-    case 5: launch_tpw<5>(p, a, st); break;
-    case 6: launch_tpw<6>(p, a, st); break;
-    case 7: launch_tpw<7>(p, a, st); break;
-    case 8: launch_tpw<8>(p, a, st); break;
-    default: return hipErrorInvalidValue;
-    }
+    if (!(p.bf16 ? launch_fused_t<true>(p, a, st) : launch_fused_t<false>(p, a, st))) return hipErrorInvalidValue;
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     return launch_finalize(a, st);

@@ -29,7 +29,7 @@ namespace fcs {
 // ------------------------------------------------------------------------------------
 // WAVES = 4 or 8 waves per block: a block covers WAVES * QW query rows and streams its keys
 // once, so taller blocks divide the key traffic of this pass.
-template <int D, int QW, int WAVES>
+template <int D, int QW, int WAVES, bool BF>
 __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args a)
 {
     constexpr int THREADS = 64 * WAVES;
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
                 for (int t = 0; t < NT; ++t)
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb)
-                        cn[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t], qf[nb][t], cn[nb], 0, 0, 0);
+                        cn[nb] = mfma16<BF>(af[t], qf[nb][t], cn[nb]);
                 // the new MFMAs are in the instruction stream before the old scores are touched
                 if (NB == 2)
                     asm volatile("" : "+v"(cn[0]), "+v"(cn[NB - 1]), "+v"(cp[0]), "+v"(cp[NB - 1]));
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
                 floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int t = 0; t < NT; ++t)
-                    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t], qf[nb][t], c, 0, 0, 0);
+                    c = mfma16<BF>(af[t], qf[nb][t], c);
                 acc[na][nb] = c;
             }
         }
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(64) void fcs_merge_stats_kernel(const Args a)
 // ------------------------------------------------------------------------------------
 // pass 2: column sums of p_ij = 2^(c*s_ij - lse2[i])
 // ------------------------------------------------------------------------------------
-template <int D, int KW>
+template <int D, int KW, bool BF>
 __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
 {
     constexpr int NA = KW / 32;
@@ -414,7 +414,7 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
             for (int tt = 0; tt < NT; ++tt)
 #pragma unroll
                 for (int na = 0; na < NA; ++na)
-                    cn[na] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[na][tt], bf[tt], cn[na], 0, 0, 0);
+                    cn[na] = mfma16<BF>(kf[na][tt], bf[tt], cn[na]);
 #pragma unroll
             for (int na = 0; na < NA; ++na) {
                 if (!edge) {
@@ -494,18 +494,18 @@ hipError_t launch_finalize(const Args &a, hipStream_t st)
     return hipGetLastError();
 }
 
-template <int D>
+template <int D, bool BF>
 static hipError_t launch_d(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 blk(256);
     {
         const dim3 grid(p.n_qblk, p.n_chunks, p.B * p.H);
         if (p.qw == 64 && p.k1_waves == 8)
-            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64, 8>), grid, dim3(512), 0, st, a);
+            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64, 8, BF>), grid, dim3(512), 0, st, a);
         else if (p.qw == 64)
-            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64, 4>), grid, blk, 0, st, a);
+            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64, 4, BF>), grid, blk, 0, st, a);
         else
-            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 32, 4>), grid, blk, 0, st, a);
+            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 32, 4, BF>), grid, blk, 0, st, a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -518,9 +518,9 @@ static hipError_t launch_d(const Plan &p, const Args &a, hipStream_t st)
     {
         const dim3 grid(p.n_kblk, p.gh * p.gq, p.B);
         if (p.kw == 64)
-            hipLaunchKernelGGL((fcs_colsum_kernel<D, 64>), grid, blk, 0, st, a);
+            hipLaunchKernelGGL((fcs_colsum_kernel<D, 64, BF>), grid, blk, 0, st, a);
         else
-            hipLaunchKernelGGL((fcs_colsum_kernel<D, 32>), grid, blk, 0, st, a);
+            hipLaunchKernelGGL((fcs_colsum_kernel<D, 32, BF>), grid, blk, 0, st, a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -536,7 +536,11 @@ int launch_colsum(const Plan &p, const Args &a, void *stream)
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (p.fewrows) return (int)launch_fewrows(p, a, st);
     if (p.fused) return (int)launch_fused(p, a, st);
-    hipError_t e = (p.D == 64) ? launch_d<64>(p, a, st) : launch_d<128>(p, a, st);
+    hipError_t e;
+    if (p.bf16)
+        e = (p.D == 64) ? launch_d<64, true>(p, a, st) : launch_d<128, true>(p, a, st);
+    else
+        e = (p.D == 64) ? launch_d<64, false>(p, a, st) : launch_d<128, false>(p, a, st);
     return (int)e;
 }
 

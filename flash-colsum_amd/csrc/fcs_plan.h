@@ -17,6 +17,7 @@ constexpr int kTargetBlocks = 1024; // 256 CUs x 4: enough workgroups to fill th
 
 struct Plan {
     int B, H, Sq, Sk, D;
+    int bf16;    // operands are bf16 instead of fp16 (set by the caller after make_plan)
     int q_rows;  // query rows that are averaged: min(cls_n, Sq) or Sq
     int causal, k_past;
     // pass 1: row statistics.  grid = (n_qblk, n_chunks, B*H)
@@ -55,6 +56,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
 {
     if (B < 1 || H < 1 || Sq < 1 || Sk < 1 || D < 1 || k_past < 0) return false;
     p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk; p.D = D;
+    p.bf16 = 0;
     p.causal = causal ? 1 : 0;
     p.k_past = causal ? k_past : 0;
     p.q_rows = (!causal && cls_n > 0 && cls_n < Sq) ? cls_n : Sq;

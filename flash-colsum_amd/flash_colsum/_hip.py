@@ -16,7 +16,7 @@ from typing import Optional
 import torch
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libflashcolsum.so")
-_ABI_VERSION = 2
+_ABI_VERSION = 3
 _lib = None
 
 _I64x4 = ctypes.c_int64 * 4
@@ -38,18 +38,20 @@ def lib() -> ctypes.CDLL:
         cdll.fcs_strerror.argtypes = [ctypes.c_int]
         cdll.fcs_workspace_bytes.restype = ctypes.c_size_t
         cdll.fcs_workspace_bytes.argtypes = [ctypes.c_int] * 7
-        cdll.fcs_colsum_noncausal_f16.restype = ctypes.c_int
-        cdll.fcs_colsum_noncausal_f16.argtypes = [
-            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
-            ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-            ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
-            ctypes.c_float, ctypes.c_int, ctypes.c_void_p]
-        cdll.fcs_colsum_causal_f16.restype = ctypes.c_int
-        cdll.fcs_colsum_causal_f16.argtypes = [
-            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
-            ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-            ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
-            ctypes.c_float, ctypes.c_void_p]
+        for fn in (cdll.fcs_colsum_noncausal_f16, cdll.fcs_colsum_noncausal_bf16):
+            fn.restype = ctypes.c_int
+            fn.argtypes = [
+                ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
+                ctypes.c_float, ctypes.c_int, ctypes.c_void_p]
+        for fn in (cdll.fcs_colsum_causal_f16, cdll.fcs_colsum_causal_bf16):
+            fn.restype = ctypes.c_int
+            fn.argtypes = [
+                ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
+                ctypes.c_float, ctypes.c_void_p]
         got = cdll.fcs_abi_version()
         if got != _ABI_VERSION:
             raise RuntimeError(f"libflashcolsum.so has ABI {got}, this host layer needs {_ABI_VERSION}")
@@ -66,10 +68,10 @@ def _check(code: int, what: str) -> None:
         raise RuntimeError(f"{what} failed with code {code}: {strerror(code)}")
 
 
-def _as_kernel_input(t: torch.Tensor) -> torch.Tensor:
-    """fp16, unit last stride, 16-byte aligned rows/heads/base; copies only when it must."""
-    if t.dtype != torch.float16:
-        t = t.to(torch.float16)
+def _as_kernel_input(t: torch.Tensor, dtype: torch.dtype = torch.float16) -> torch.Tensor:
+    """`dtype` (fp16 or bf16), unit last stride, 16-byte aligned rows/heads/base; copies only when it must."""
+    if t.dtype != dtype:
+        t = t.to(dtype)
     ok = (
         t.stride(3) == 1
         and t.stride(2) % 8 == 0
@@ -124,15 +126,16 @@ def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16):
     stream = torch.cuda.current_stream(dev).cuda_stream
     ws = _workspace(dev, stream, n_ws)
     qs, ks = _I64x4(*q.stride()), _I64x4(*k.stride())
+    bf16 = q.dtype == torch.bfloat16
     if causal:
-        rc = lib().fcs_colsum_causal_f16(
-            q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
-            h, s_q, s_k, d, int(k_past), qs, ks, float(scale), stream)
+        fn = lib().fcs_colsum_causal_bf16 if bf16 else lib().fcs_colsum_causal_f16
+        rc = fn(q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
+                h, s_q, s_k, d, int(k_past), qs, ks, float(scale), stream)
     else:
-        rc = lib().fcs_colsum_noncausal_f16(
-            q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
-            b, h, s_q, d, qs, ks, float(scale), int(cls_n), stream)
-    _check(rc, "fcs_colsum_causal_f16" if causal else "fcs_colsum_noncausal_f16")
+        fn = lib().fcs_colsum_noncausal_bf16 if bf16 else lib().fcs_colsum_noncausal_f16
+        rc = fn(q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
+                b, h, s_q, d, qs, ks, float(scale), int(cls_n), stream)
+    _check(rc, ("fcs_colsum_causal" if causal else "fcs_colsum_noncausal") + ("_bf16" if bf16 else "_f16"))
     return (out, out_h) if want_f16 else out
 
 
@@ -140,8 +143,10 @@ def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n:
     """Enqueue one call; returns the fp32 means, or (fp32, fp16) when `want_f16`."""
     if q.device.type != "cuda" or k.device != q.device:
         raise ValueError(f"query and key must live on the same GPU, got {q.device} and {k.device}")
-    q = _as_kernel_input(q)
-    k = _as_kernel_input(k)
+    # bf16 inputs run natively when both are bf16; every other dtype is converted to fp16
+    dtype = torch.bfloat16 if (q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16) else torch.float16
+    q = _as_kernel_input(q, dtype)
+    k = _as_kernel_input(k, dtype)
     if q.device.index == torch.cuda.current_device():
         return _enqueue(causal, q, k, scale, cls_n, k_past, want_f16)
     with torch.cuda.device(q.device):

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FCS_ABI_VERSION 2
+#define FCS_ABI_VERSION 3
 
 enum {
     FCS_OK = 0,
@@ -82,6 +82,21 @@ int fcs_colsum_causal_f16(const void *q, const void *k, float *out, void *out_f1
                           int H, int Q_len, int K_len, int D, int k_past,
                           const int64_t q_strides[4], const int64_t k_strides[4],
                           float scale, void *hip_stream);
+
+/* The same two launch functions for bf16 inputs: q and k hold bfloat16 values (same shapes,
+ * strides in elements, alignment rules, workspace size and outputs as above; `out_f16` is still
+ * IEEE fp16, the reference's result dtype for every input dtype).  Products are exact and
+ * accumulated in fp32, like the reference kernels, which upcast their operands before the
+ * dot product (reference: flash_colsum/kernel_noncausal_batched.py:37,54,
+ * flash_colsum/kernel_causal.py:32,52). */
+int fcs_colsum_noncausal_bf16(const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes,
+                              int B, int H, int S, int D,
+                              const int64_t q_strides[4], const int64_t k_strides[4],
+                              float scale, int cls_n, void *hip_stream);
+int fcs_colsum_causal_bf16(const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes,
+                           int H, int Q_len, int K_len, int D, int k_past,
+                           const int64_t q_strides[4], const int64_t k_strides[4],
+                           float scale, void *hip_stream);
 
 #ifdef __cplusplus
 }

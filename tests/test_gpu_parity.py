@@ -255,6 +255,49 @@ def test_prescaled_shared_q_variant(shape, same, kw, boost):
     _assert_close(_run(q, k, **kw), _oracle(q, k, **kw), f"prescaled {shape} same={same} {kw} boost={boost}")
 
 
+@pytest.mark.parametrize("qs,ks,kw", [
+    ((4, 8, 512, 64), (4, 8, 512, 64), {}),                          # fused, whole tiles
+    ((8, 2, 2048, 64), (8, 2, 2048, 64), {}),                        # fused, where fp16 would take the pre-scaled variant
+    ((2, 3, 577, 64), (2, 3, 577, 64), {}),                          # fused, ragged
+    ((2, 3, 577, 64), (2, 3, 577, 64), {"scale": 40.0}),             # ... max-subtracted fallback
+    ((2, 2, 300, 128), (2, 2, 300, 128), {"scale": -0.1}),           # two-pass, D = 128
+    ((1, 4, 4096, 64), (1, 4, 4096, 64), {}),                        # two-pass, split keys
+    ((1, 8, 128, 128), (1, 8, 4096, 128), {"is_causal": True}),
+    ((1, 4, 100, 64), (1, 4, 1000, 64), {"is_causal": True}),
+    ((3, 5, 577, 64), (3, 5, 577, 64), {"cls_len": 1}),              # few-rows
+    ((2, 3, 333, 128), (2, 3, 333, 128), {"cls_len": 3}),
+])
+def test_bf16_inputs_run_natively(qs, ks, kw):
+    """bf16 operands (reference: the Triton kernels upcast them before the dot product,
+    kernel_noncausal_batched.py:37,54): the oracle gets the same bf16-rounded values."""
+    from flash_colsum import flash_colsum
+
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(qs, generator=g).bfloat16()
+    k = torch.randn(ks, generator=g).bfloat16()
+    # values far outside fp16's range, which a conversion to fp16 would destroy
+    q[..., 0] *= 2.0 ** 40
+    k[..., 0] *= 2.0 ** -40
+    out = _run(q, k, **kw)
+    ref = _oracle(q.float(), k.float(), **kw)
+    _assert_close(out, ref, f"bf16 {qs} {ks} {kw}")
+    h = flash_colsum(q.cuda(), k.cuda(), **kw)
+    assert h.dtype == torch.float16 and torch.equal(h, out.half())
+
+
+def test_other_input_dtypes_are_converted_to_fp16():
+    from flash_colsum import flash_colsum_f32
+
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn((2, 4, 200, 64), generator=g)
+    k = torch.randn((2, 4, 200, 64), generator=g)
+    ref = _oracle(q.half(), k.half())
+    _assert_close(flash_colsum_f32(q.cuda(), k.cuda()), ref, "fp32 inputs")
+    _assert_close(flash_colsum_f32(q.cuda().double(), k.cuda().half()), ref, "fp64 / fp16 inputs")
+    _assert_close(flash_colsum_f32(q.half().bfloat16().cuda(), k.half().cuda()),
+                  _oracle(q.half().bfloat16().half(), k.half()), "bf16 / fp16 inputs")
+
+
 def test_explicit_k_past():
     """The causal launcher's K_past argument (reference: kernel_causal.py:94-113)."""
     from flash_colsum import _hip

@@ -61,11 +61,11 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _hip.lib()
     names = _declared_symbols()
-    assert names == ["fcs_abi_version", "fcs_colsum_causal_f16", "fcs_colsum_noncausal_f16", "fcs_strerror",
-                     "fcs_workspace_bytes"]
+    assert names == ["fcs_abi_version", "fcs_colsum_causal_bf16", "fcs_colsum_causal_f16", "fcs_colsum_noncausal_bf16",
+                     "fcs_colsum_noncausal_f16", "fcs_strerror", "fcs_workspace_bytes"]
     for n in names:
         assert getattr(lib, n) is not None
-    assert lib.fcs_abi_version() == 2
+    assert lib.fcs_abi_version() == 3
 
 
 def test_strerror_is_total():
@@ -107,6 +107,13 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert ca(p, p, p, None, p, 1 << 30, 8, 16, 64, 64, -1, st, st, 0.125, None) == -2
     assert ca(p, p, p, None, p, 1 << 30, 8, 16, 64, 96, 48, st, st, 0.125, None) == -3
     assert ca(p, p, p, None, p, 16, 8, 16, 64, 64, 48, st, st, 0.125, None) == -5
+    # the bf16 entry points share the checks
+    nb, cb = lib.fcs_colsum_noncausal_bf16, lib.fcs_colsum_causal_bf16
+    assert nb(None, p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
+    assert nb(p, p, p, None, p, 1 << 30, 2, 8, 16, 80, st, st, 0.125, -1, None) == -3
+    assert nb(p, p, p, None, p, 16, 2, 8, 16, 64, st, st, 0.125, -1, None) == -5
+    assert cb(p, p, p, None, p, 1 << 30, 8, 16, 64, 64, -1, st, st, 0.125, None) == -2
+    assert cb(p, p, p, None, p, 16, 8, 16, 64, 64, 48, st, st, 0.125, None) == -5
 
 
 def test_missing_library_is_loud(monkeypatch, tmp_path):
