@@ -20,6 +20,7 @@ _ABI_VERSION = 3
 _lib = None
 
 _I64x4 = ctypes.c_int64 * 4
+_HEAD_DIMS = (64, 128)  # head dims the library is compiled for
 
 
 def lib() -> ctypes.CDLL:
@@ -145,6 +146,13 @@ def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n:
         raise ValueError(f"query and key must live on the same GPU, got {q.device} and {k.device}")
     # bf16 inputs run natively when both are bf16; every other dtype is converted to fp16
     dtype = torch.bfloat16 if (q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16) else torch.float16
+    # the kernels are compiled for head dims 64 and 128: smaller ones are padded with zero channels
+    # (a copy), which leaves every score unchanged; the caller's scale already reflects the real D
+    d = q.shape[-1]
+    if d not in _HEAD_DIMS and d < _HEAD_DIMS[-1] and d == k.shape[-1]:
+        pad = next(x for x in _HEAD_DIMS if x > d) - d
+        q = torch.nn.functional.pad(q.to(dtype), (0, pad))
+        k = torch.nn.functional.pad(k.to(dtype), (0, pad))
     q = _as_kernel_input(q, dtype)
     k = _as_kernel_input(k, dtype)
     if q.device.index == torch.cuda.current_device():

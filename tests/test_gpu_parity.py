@@ -186,8 +186,8 @@ def test_reference_error_handling():
     with pytest.raises(ValueError, match="same shape"):
         flash_colsum(q, k)
     with pytest.raises(RuntimeError, match="head dim"):
-        flash_colsum(torch.randn(1, 2, 16, 48, device="cuda", dtype=torch.float16),
-                     torch.randn(1, 2, 16, 48, device="cuda", dtype=torch.float16))
+        flash_colsum(torch.randn(1, 2, 16, 160, device="cuda", dtype=torch.float16),
+                     torch.randn(1, 2, 16, 160, device="cuda", dtype=torch.float16))
 
 
 # ---------------------------------------------------------------------------------------
@@ -296,6 +296,16 @@ def test_other_input_dtypes_are_converted_to_fp16():
     _assert_close(flash_colsum_f32(q.cuda().double(), k.cuda().half()), ref, "fp64 / fp16 inputs")
     _assert_close(flash_colsum_f32(q.half().bfloat16().cuda(), k.half().cuda()),
                   _oracle(q.half().bfloat16().half(), k.half()), "bf16 / fp16 inputs")
+
+
+@pytest.mark.parametrize("d", [8, 32, 40, 80, 96])
+def test_other_head_dims_are_zero_padded(d):
+    q, k = _inputs((2, 3, 150, d), (2, 3, 150, d), seed=7)
+    _assert_close(_run(q, k), _oracle(q, k), f"D={d}")
+    q, k = _inputs((1, 3, 50, d), (1, 3, 400, d), seed=8)
+    _assert_close(_run(q, k, is_causal=True), _oracle(q, k, is_causal=True), f"causal D={d}")
+    with pytest.raises(RuntimeError, match="head dim"):
+        _run(*_inputs((1, 2, 16, 136), (1, 2, 16, 136)))
 
 
 def test_explicit_k_past():
