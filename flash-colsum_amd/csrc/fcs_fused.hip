@@ -378,6 +378,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         // ---------------- phase 1: one step per key tile
 #pragma unroll
         for (int t = 0; t < TPW; ++t) {
+            // The two waves that share a SIMD (w and w + 4) take turns at the higher issue priority, one
+            // key tile each.  With equal priorities the older wave wins every arbitration, finishes
+            // its tiles ~20 % early and idles at the barrier while the other one runs alone, without
+            // anything to overlap its MFMAs with (measured: 2-3 % of the kernel).
+            if (((t & 1) != 0) == (wave >= 4)) asm volatile("s_setprio 2");
+            else asm volatile("s_setprio 0");
             // the operands of this tile were read back during the previous step: they have landed,
             // their ring slots are free again and take the look-ahead fetches
             if (t == 0) {
