@@ -308,6 +308,38 @@ def test_other_head_dims_are_zero_padded(d):
         _run(*_inputs((1, 2, 16, 136), (1, 2, 16, 136)))
 
 
+def test_random_shapes_every_path():
+    """60 seeded random shapes, scales, modes and dtypes: whichever kernel the plan picks must
+    agree with the oracle."""
+    import random
+
+    rng = random.Random(1234)
+    for case in range(60):
+        d = rng.choice([64, 64, 128, 32, 96])
+        h = rng.randint(1, 6)
+        mode = rng.choice(["plain", "plain", "cls", "causal"])
+        if mode == "causal":
+            b, sq, sk = 1, rng.randint(1, 300), rng.randint(1, 3000)
+        else:
+            b = rng.randint(1, 5)
+            sq = sk = rng.choice([rng.randint(1, 100), rng.randint(100, 700), rng.randint(700, 2500), rng.randint(2049, 5000)])
+        kw = {}
+        if mode == "causal":
+            kw["is_causal"] = True
+        if mode == "cls":
+            kw["cls_len"] = rng.choice([1, 2, 3, 4, 5, 17, 64, sq, sq + 3])
+        if rng.random() < 0.5:
+            kw["scale"] = rng.choice([0.05, 0.125, 0.3, -0.1, 1.0, 3.0])
+        bf16 = rng.random() < 0.3
+        g = torch.Generator().manual_seed(1000 + case)
+        q = torch.randn((b, h, sq, d), generator=g)
+        k = torch.randn((b, h, sk, d), generator=g)
+        q, k = (q.bfloat16(), k.bfloat16()) if bf16 else (q.half(), k.half())
+        what = f"case {case}: q{tuple(q.shape)} k{tuple(k.shape)} {kw} {'bf16' if bf16 else 'fp16'}"
+        print(what, flush=True)
+        _assert_close(_run(q, k, **kw), _oracle(q.float(), k.float(), **kw), what)
+
+
 def test_explicit_k_past():
     """The causal launcher's K_past argument (reference: kernel_causal.py:94-113)."""
     from flash_colsum import _hip
