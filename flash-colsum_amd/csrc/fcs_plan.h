@@ -10,6 +10,7 @@ namespace fcs {
 constexpr int kWavesPerBlock = 4;   // 256 threads
 constexpr int kStageKeys = 64;      // keys staged in LDS per step of the row-statistics pass
 constexpr int kStageRows = 64;      // query rows staged in LDS per step of the column pass
+constexpr int kComputeUnits = 256;  // MI355X
 constexpr int kFusedMaxKeys = 2048; // 8 waves x 8 tiles x 32 keys of fp32 scores per 32 query rows
 constexpr int kFewRowsMaxRows = 4;      // few-rows path: at most this many averaged query rows per head ...
 constexpr int kFewRowsMaxScores = 12288; // ... and rows * Sk scores (48 KB of LDS)
@@ -68,7 +69,11 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     p.n_qblk = ceil_div(p.q_rows, qblk);
     p.rows_pad = p.n_qblk * qblk;
     const long base1 = (long)p.n_qblk * B * H;
-    int want = (int)((kTargetBlocks + base1 - 1) / base1);
+    // One generation of workgroups: an 8-wave block fills a compute unit's registers, the 4-wave
+    // blocks fit twice.  Every further generation pays the block start (Q fragments, first key
+    // stage: ~5 us) again, which nothing overlaps.
+    const int target1 = (p.k1_waves == 8) ? kComputeUnits : 2 * kComputeUnits;
+    int want = (int)((target1 + base1 - 1) / base1);
     int max_chunks = ceil_div(Sk, 4 * kStageKeys);  // at least 256 keys per split
     if (want > max_chunks) want = max_chunks;
     if (want < 1) want = 1;
@@ -80,17 +85,36 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     p.kw = ((long)ceil_div(Sk, 256) * B >= kTargetBlocks / 4) ? 64 : 32;
     const int kblk = kWavesPerBlock * p.kw;
     p.n_kblk = ceil_div(Sk, kblk);
+    // Groups along heads and along staged query tiles, chosen by a small cost model in units of
+    // one stage (64 query rows against the block's keys): a block pays for its stages, for each
+    // head's key fragments, and for starting and finishing; blocks run in generations of as many
+    // as the GPU holds at once (registers allow 4 / 2 blocks per compute unit at D = 64, 3 / 2 at
+    // D = 128 for 32 / 64 keys per wave).
     const long base2 = (long)p.n_kblk * B;
-    int g = (int)((kTargetBlocks + base2 - 1) / base2);
-    if (g < 1) g = 1;
-    p.gh = g < H ? g : H;
-    p.heads_per_group = ceil_div(H, p.gh);
-    p.gh = ceil_div(H, p.heads_per_group);
-    int gq = ceil_div(g, p.gh);
-    if (gq > n_qt) gq = n_qt;
-    if (gq < 1) gq = 1;
-    p.qtiles_per_group = ceil_div(n_qt, gq);
-    p.gq = ceil_div(n_qt, p.qtiles_per_group);
+    const int per_cu = (p.kw == 64) ? 2 : (D == 64 ? 4 : 3);
+    const long resident = (long)kComputeUnits * per_cu;
+    double best = 0.;
+    p.gh = 1; p.gq = 1; p.heads_per_group = H; p.qtiles_per_group = n_qt;
+    bool first = true;
+    for (int hpg = 1; hpg <= H; hpg = (hpg < 4) ? hpg + 1 : hpg + hpg / 2) {
+        const int gh = ceil_div(H, hpg);
+        const int hpg_e = ceil_div(H, gh);
+        for (int gen = 0; gen <= 2; ++gen) {  // query groups: none, or enough for one / two generations
+            long gq = (gen == 0) ? 1 : (resident * gen + base2 * gh - 1) / (base2 * gh);
+            if (gq > n_qt) gq = n_qt;
+            if (gq < 1) gq = 1;
+            const int tpg = ceil_div(n_qt, (int)gq);
+            const int gq_e = ceil_div(n_qt, tpg);
+            const long blocks = base2 * gh * gq_e;
+            const double gens = (double)((blocks + resident - 1) / resident);
+            const double cost = gens * (hpg_e * (tpg + 1.0) + 3.0) + 0.02 * gh * gq_e;
+            if (first || cost < best) {
+                first = false;
+                best = cost;
+                p.gh = gh; p.heads_per_group = hpg_e; p.gq = gq_e; p.qtiles_per_group = tpg;
+            }
+        }
+    }
 
     // ---- few-rows path: a batch of matrix-vector products, one workgroup per (batch entry, head group)
     p.fewrows = 0;
