@@ -98,20 +98,24 @@ __device__ __forceinline__ bool reduce_rows(const float (&v)[16], RowRed &rr, in
     const int pbase = (qg * 32 + row) * kg_n;
     if (half == 0) part[pbase + kg] = s;
     __syncthreads();
-    float tot = part[pbase];
-    if (kg_n > 1) tot = MAX ? fmaxf(tot, part[pbase + 1]) : tot + part[pbase + 1];
-    if (kg_n > 2) {
-        const float t2 = part[pbase + 2], t3 = part[pbase + 3];
-        tot = MAX ? fmaxf(tot, fmaxf(t2, t3)) : tot + (t2 + t3);
-    }
-    if (kg_n > 4) {
-        const float t4 = part[pbase + 4], t5 = part[pbase + 5], t6 = part[pbase + 6], t7 = part[pbase + 7];
-        tot = MAX ? fmaxf(tot, fmaxf(fmaxf(t4, t5), fmaxf(t6, t7))) : tot + ((t4 + t5) + (t6 + t7));
-    }
+    float tot;
     bool out_of_range = false;
+    // every wave looks at all 256 partials of the workgroup: lane L at floats [4L, 4L + 4)
+    const floatx4 f = reinterpret_cast<const floatx4 *>(part)[lane];
+    if (kg_n == 8) {
+        // those four are key groups 4*half .. 4*half + 3 of this lane's own row: its neighbour holds the rest
+        const float own = MAX ? fmaxf(fmaxf(f[0], f[1]), fmaxf(f[2], f[3])) : (f[0] + f[1]) + (f[2] + f[3]);
+        const float other = dpp_get<kDppXor1>(own);
+        tot = MAX ? fmaxf(own, other) : own + other;
+    } else {
+        tot = part[pbase];
+        if (kg_n > 1) tot = MAX ? fmaxf(tot, part[pbase + 1]) : tot + part[pbase + 1];
+        if (kg_n > 2) {
+            const float t2 = part[pbase + 2], t3 = part[pbase + 3];
+            tot = MAX ? fmaxf(tot, fmaxf(t2, t3)) : tot + (t2 + t3);
+        }
+    }
     if (!MAX) {
-        // every wave looks at all 256 partials of the workgroup: lane L at floats [4L, 4L + 4)
-        const floatx4 f = reinterpret_cast<const floatx4 *>(part)[lane];
         const bool hi = !(f[0] < sum_hi) || !(f[1] < sum_hi) || !(f[2] < sum_hi) || !(f[3] < sum_hi);
         const float m01 = fmaxf(f[0], f[1]), m23 = fmaxf(f[2], f[3]);
         float lowest;  // smallest per-row maximum over key groups among the rows this lane sees
@@ -346,7 +350,9 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 
     for (int unit = 0; unit < n_units; ++unit) {
         const int h = h_begin + unit;
-        // this head's Q tile and first key tile (fetched during the previous head)
+        // this head's Q tile and first key tile (fetched during the previous head).  (Reading them
+        // back earlier, under the previous head's column-sum FMAs, makes them live across the loop
+        // and the kernel spills.)
         if (PRE) {
             take_q_shared(unit & 1, qf);
         } else {
