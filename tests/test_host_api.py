@@ -86,6 +86,32 @@ def test_workspace_bytes():
     assert wb(True, 1, 32, 512, 65536, 128) < 64 << 20
 
 
+def test_workspace_plan_over_random_shapes():
+    """The launch plan behind fcs_workspace_bytes() must hold for any shape: aligned, nonzero,
+    linear in the sequence lengths (never quadratic), and independent of cls_n beyond its clamp."""
+    import random
+
+    rng = random.Random(7)
+    wb = _hip.workspace_bytes
+    for _ in range(400):
+        causal = rng.random() < 0.4
+        b = 1 if causal else rng.choice([1, 2, 7, 32, 300])
+        h = rng.choice([1, 2, 8, 16, 32, 40])
+        if b * h > 65535:
+            continue
+        d = rng.choice([64, 128])
+        sk = rng.choice([1, 5, 64, 577, 2048, 2049, 8191, 65536, 262144])
+        sq = rng.choice([1, 16, 128, 512, 1000]) if causal else sk
+        cls_n = -1 if causal else rng.choice([-1, 1, 2, 4, 5, 100, sq, sq + 7])
+        n = wb(causal, b, h, sq, sk, d, cls_n)
+        assert n > 0 and n % 256 == 0, (causal, b, h, sq, sk, d, cls_n, n)
+        # a few floats per (batch, head, row) plus at most a few thousand partial rows of Sk floats
+        bound = 64 * b * h * (sq + 1024) + 4 * 4096 * (b * sk + 1024) + (1 << 20)
+        assert n <= bound, (causal, b, h, sq, sk, d, cls_n, n, bound)
+        if cls_n >= sq:
+            assert n == wb(causal, b, h, sq, sk, d, -1)
+
+
 def test_argument_errors_are_reported_without_a_gpu():
     lib = _hip.lib()
     st = (ctypes.c_int64 * 4)(8 * 16 * 64, 16 * 64, 64, 1)
