@@ -148,14 +148,15 @@ __device__ __forceinline__ floatx4 row_values(const RowRed &rr, int i4, int g)
 //                 no padding keys anywhere, and tile addresses need no per-lane arithmetic.
 // RAGGED = true : anything else; fetches compute and clamp their rows per lane and every exponent
 //                 is masked per lane.
-// PRE = true (only with RAGGED = false, 8 key groups): the block's Q tile is multiplied by
+// PRE = 8 or 4 (0 = off; only with RAGGED = false and that many key groups, i.e. 1 or 2 query
+//                 groups): each query group's Q tile is multiplied by
 //                 c = scale * log2(e) in fp32 ONCE per head, rounded back to fp16 and shared by the
 //                 eight waves through LDS, so the scores leave the MFMAs already in the exponent's
 //                 unit and the per-score multiply disappears.  The extra fp16 rounding of Q perturbs
 //                 each score by ~2^-12 relative; the launcher only picks this variant when at least
 //                 4096 (head, row) pairs are averaged per output, where the effect on the means is
 //                 below 1e-4 relative (measured 6.5e-5 at B8 H16 S2048).
-template <int D, int TPW, bool RAGGED, bool PRE, bool BF>
+template <int D, int TPW, bool RAGGED, int PRE, bool BF>
 __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 {
     static_assert(D == 64, "the fused path is laid out for 64-wide heads");
@@ -171,11 +172,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     __shared__ __attribute__((aligned(16))) float red[8 * 32 * kRedPitch];
     __shared__ __attribute__((aligned(16))) float part[2 * 256];
     __shared__ __attribute__((aligned(16))) float wv[8 * 32];
-    __shared__ __attribute__((aligned(16))) char qshare[PRE ? 2 * 4096 : 16];  // pre-scaled Q tile, double-buffered
+    constexpr int PQG = PRE ? 8 / PRE : 1;  // query groups of the pre-scaled variant
+    __shared__ __attribute__((aligned(16))) char qshare[PRE ? 2 * PQG * 4096 : 16];  // pre-scaled Q tiles, double-buffered
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what derives from it stays in SGPRs
-    const int kg_n = PRE ? 8 : a.f_kg, qg_n = 8 / kg_n;  // a constant folds the reduction's branches away
+    const int kg_n = PRE ? PRE : a.f_kg, qg_n = 8 / kg_n;  // a constant folds the reduction's branches away
     const int qg = wave / kg_n, kg = wave - qg * kg_n;
     // The row blocks of one (head group, batch entry) read the same K: they run on one XCD, close
     // together in time.
@@ -291,16 +293,26 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     //     fetched into it; at most three items (12 DMA instructions) are in flight.
     //   * Past the last head the fetches repeat it, so that the number of outstanding DMA
     //     instructions at every wait is a compile-time constant.
-    // PRE: the Q item of a head is not a tile in the ring but this wave's 4 rows (512 B) of the raw
-    // tile, one ordinary 8-byte load per lane; the wave scales them and publishes them in `qshare`.
-    uint2 qraw = {0u, 0u};
+    // PRE: the Q item of a head is not a tile in the ring but this wave's 32 / PRE rows of its query
+    // group's raw tile (512 B or 1 KB), one ordinary 8- or 16-byte load per lane; the wave scales
+    // them and publishes them in `qshare`.
+    uint4v qraw = {0u, 0u, 0u, 0u};
     auto item_vm = [&](int j_ahead) { return (PRE && (j_ahead % ITEMS) == 0) ? 1 : NT; };  // VMEM instructions of an item
     auto fetch_pos_piece = [&](int h_now, int j_ahead /* item index counted from the Q tile of head h_now, compile-time */,
                                int slot, int tt) {
         const int hh = min(h_now + j_ahead / ITEMS, h_end - 1);
         const int j = j_ahead % ITEMS;
         if (j == 0 && PRE) {
-            if (tt == 0) qraw = *reinterpret_cast<const uint2 *>(q_b + (int64_t)hh * q_head_b + wave * 512 + lane * 8);
+            if (tt == 0) {
+                const char *src = q_b + (int64_t)hh * q_head_b;
+                if (PRE == 8) {
+                    const uint2 v = *reinterpret_cast<const uint2 *>(src + kg * 512 + lane * 8);
+                    qraw[0] = v.x;
+                    qraw[1] = v.y;
+                } else {
+                    qraw = *reinterpret_cast<const uint4v *>(src + kg * 1024 + lane * 16);
+                }
+            }
         } else if (j == 0)
             fetch_piece(q_b + (int64_t)hh * q_head_b, q_row_b, q_voff, a.Sq - q0, slot, tt);
         else
@@ -318,20 +330,27 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         return s_ >= NS ? s_ - NS : s_;
     };
 
-    // PRE: scale this wave's 4 raw rows by c (sign included) in fp32, round to fp16 and store them
-    // at their swizzled place in qshare[buf]; a workgroup barrier must follow before they are read
+    // PRE: scale this wave's raw rows by c (sign included) in fp32, round to fp16 and store them at
+    // their swizzled place in the query group's tile of qshare[buf]; a workgroup barrier must
+    // follow before they are read
     auto q_publish = [&](int buf) {
         const float cs = a.negate ? -a.c : a.c;
-        const half8 raw = __builtin_bit_cast(half8, uint4v{qraw.x, qraw.y, 0u, 0u});
-        _Float16 sc[4];
+        const half8 raw = __builtin_bit_cast(half8, qraw);
+        half8 sc;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) sc[e] = (_Float16)((float)raw[e] * cs);
-        const int row = wave * 4 + (lane >> 4), pc = (lane & 15) >> 1, hf = lane & 1;
-        char *dst = qshare + buf * 4096 + row * 128 + ((pc ^ ((row >> 1) & 7)) * 16) + hf * 8;
-        *reinterpret_cast<uint2 *>(dst) = __builtin_bit_cast(uint2, *reinterpret_cast<const uint64_t *>(sc));
+        for (int e = 0; e < (PRE == 8 ? 4 : 8); ++e) sc[e] = (_Float16)((float)raw[e] * cs);
+        char *tile = qshare + (buf * PQG + qg) * 4096;
+        if (PRE == 8) {  // 4 rows per wave, 8 bytes per lane
+            const int row = kg * 4 + (lane >> 4), pc = (lane & 15) >> 1, hf = lane & 1;
+            const uint4v u = __builtin_bit_cast(uint4v, sc);
+            *reinterpret_cast<uint2 *>(tile + row * 128 + ((pc ^ ((row >> 1) & 7)) * 16) + hf * 8) = uint2{u[0], u[1]};
+        } else {         // 8 rows per wave, one whole 16-byte piece per lane
+            const int row = kg * 8 + (lane >> 3), pc = lane & 7;
+            *reinterpret_cast<half8 *>(tile + row * 128 + ((pc ^ ((row >> 1) & 7)) * 16)) = sc;
+        }
     };
     auto take_q_shared = [&](int buf, half8 (&dst)[NT]) {
-        const uint32_t diff = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)qshare + (uint32_t)(buf * 4096) -
+        const uint32_t diff = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)qshare + (uint32_t)((buf * PQG + qg) * 4096) -
                               (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)my_ring;
         const uint32_t ta0 = take_addr[0] + diff, ta1 = take_addr[1] + diff, ta2 = take_addr[2] + diff, ta3 = take_addr[3] + diff;
         asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"
@@ -534,12 +553,15 @@ static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.f_nqblk * p.B, p.f_hg);  // x = batch entry * f_nqblk + row block
     const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
-    if (!BF && TPW == 8 && whole && p.f_kg == 8 && (long)p.H * p.q_rows >= 4096 && fabsf(a.c) <= 0.1251f * 1.44269504f)
-        hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, true, false>), grid, dim3(512), 0, st, a);
+    const bool pre = !BF && TPW == 8 && whole && (long)p.H * p.q_rows >= 4096 && fabsf(a.c) <= 0.1251f * 1.44269504f;
+    if (pre && p.f_kg == 8)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 8, false>), grid, dim3(512), 0, st, a);
+    else if (pre && p.f_kg == 4)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 4, false>), grid, dim3(512), 0, st, a);
     else if (whole)
-        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false, false, BF>), grid, dim3(512), 0, st, a);
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false, 0, BF>), grid, dim3(512), 0, st, a);
     else
-        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true, false, BF>), grid, dim3(512), 0, st, a);
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true, 0, BF>), grid, dim3(512), 0, st, a);
 }
 
 template <bool BF>

@@ -242,9 +242,13 @@ def test_edge_shapes(qs, ks, kw):
     ((1, 4, 2048, 64), False, {"scale": 0.126}, 0.0),    # just above the variant's scale limit
     ((1, 4, 2048, 64), False, {}, 6.0),                  # one head's scores exceed the variant's ceiling
     ((1, 4, 2048, 64), True, {}, 40.0),                  # ... and the unstabilised range altogether
+    ((2, 4, 1024, 64), False, {}, 0.0),                  # S = 1024: two query groups of four key groups
+    ((2, 4, 1024, 64), True, {"scale": -0.125}, 0.0),
+    ((1, 8, 1024, 64), False, {}, 6.0),
+    ((3, 4, 1024, 64), True, {}, 40.0),
 ])
 def test_prescaled_shared_q_variant(shape, same, kw, boost):
-    """Whole-tile S = 2048, D = 64 launches with >= 4096 averaged (head, row) pairs and
+    """Whole-tile S = 2048 or 1024, D = 64 launches with >= 4096 averaged (head, row) pairs and
     scale <= 1/8 run the fused kernel that scales Q once per head and rounds it to fp16;
     heads whose row sums reach 2^28 must fall back to the exact path inside that kernel."""
     q, k = _inputs(shape, shape, seed=11, same=same)
