@@ -344,6 +344,48 @@ def test_random_shapes_every_path():
         _assert_close(_run(q, k, **kw), _oracle(q.float(), k.float(), **kw), what)
 
 
+def test_two_streams_and_graph_replay():
+    """The library keeps no mutable global state and never allocates or synchronises: calls on
+    two streams may interleave, and a call can be captured into a HIP graph and replayed."""
+    from flash_colsum import flash_colsum_f32
+
+    q1, k1 = _inputs((2, 4, 700, 64), (2, 4, 700, 64), seed=21)
+    q2, k2 = _inputs((1, 4, 96, 128), (1, 4, 3000, 128), seed=22)
+    ref1, ref2 = _oracle(q1, k1), _oracle(q2, k2, is_causal=True)
+    q1, k1, q2, k2 = q1.cuda(), k1.cuda(), q2.cuda(), k2.cuda()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    outs1, outs2 = [], []
+    for _ in range(5):
+        with torch.cuda.stream(s1):
+            outs1.append(flash_colsum_f32(q1, k1))
+        with torch.cuda.stream(s2):
+            outs2.append(flash_colsum_f32(q2, k2, is_causal=True))
+    torch.cuda.synchronize()
+    for o in outs1:
+        _assert_close(o, ref1, "stream 1")
+        assert torch.equal(o, outs1[0])
+    for o in outs2:
+        _assert_close(o, ref2, "stream 2")
+        assert torch.equal(o, outs2[0])
+
+    # graph capture of one call (output and workspace come from the graph's pool), replayed with
+    # eager work and synchronisations in between; every replay must reproduce the eager result
+    eager = flash_colsum_f32(q1, k1)
+    torch.cuda.synchronize()
+    static_q = q1.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = flash_colsum_f32(static_q, k1)
+    for i in range(4):
+        static_q.copy_(q1 if i % 2 == 0 else q1.flip(2))
+        graph.replay()
+        torch.cuda.synchronize()
+        want = eager if i % 2 == 0 else flash_colsum_f32(q1.flip(2), k1)
+        torch.cuda.synchronize()
+        assert torch.equal(captured, want), f"replay {i}"
+
+
 def test_explicit_k_past():
     """The causal launcher's K_past argument (reference: kernel_causal.py:94-113)."""
     from flash_colsum import _hip
