@@ -118,10 +118,14 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
 #pragma unroll
                     for (int i = 0; i < 16; ++i) lacc[nb][i & 3] += fast_exp2(cp[nb][i] * a.c);
                 } else {
+                    // the key indices are formed inside this branch (opaque base), or the compiler
+                    // computes all sixteen ahead of the branch on every group
+                    int kb_e = p_kb + 4 * g;
+                    asm volatile("" : "+v"(kb_e));
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const float e = fast_exp2(cp[nb][i] * a.c);
-                        lacc[nb][i & 3] += (p_kb + acc_row(i, g) <= thr[nb]) ? e : 0.f;
+                        lacc[nb][i & 3] += (kb_e + (8 * (i >> 2) + (i & 3)) <= thr[nb]) ? e : 0.f;
                     }
                 }
             }
@@ -421,10 +425,12 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) colacc[na][i] += fast_exp2(fmaf(cn[na][i], a.c, nlse));
                 } else {
+                    int kb_e = kw0 + na * 32 + 4 * g;  // opaque: keeps the key indices inside this branch
+                    asm volatile("" : "+v"(kb_e));
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const float p = fast_exp2(fmaf(cn[na][i], a.c, nlse));
-                        colacc[na][i] += (kw0 + na * 32 + acc_row(i, g) <= lim) ? p : 0.f;
+                        colacc[na][i] += (kb_e + (8 * (i >> 2) + (i & 3)) <= lim) ? p : 0.f;
                     }
                 }
             }
