@@ -418,6 +418,24 @@ def test_strided_and_unaligned_inputs():
                   _oracle(every_other[:, :, ::2].cpu(), every_other[:, :, ::2].cpu()), "row stride 2*D")
 
 
+def test_strided_inputs_on_every_path():
+    """(B, S, H, D) storage viewed as (B, H, S, D) (rows H*D apart, no copy) through the few-rows,
+    whole-tile fused, two-pass and causal kernels."""
+    g = torch.Generator().manual_seed(9)
+
+    def bshd(b, s, h, d):
+        t = torch.randn((b, s, h, d), generator=g).half()
+        return t.cuda().permute(0, 2, 1, 3), t.permute(0, 2, 1, 3)
+
+    for (b, s, h, d, kw) in [(2, 333, 3, 64, {"cls_len": 2}), (2, 1024, 4, 64, {}), (1, 2500, 2, 64, {}),
+                             (2, 200, 3, 128, {})]:
+        (q, q_cpu), (k, k_cpu) = bshd(b, s, h, d), bshd(b, s, h, d)
+        assert not q.is_contiguous()
+        _assert_close(_run(q, k, **kw), _oracle(q_cpu, k_cpu, **kw), f"strided {b, s, h, d} {kw}")
+    (q, q_cpu), (k, k_cpu) = bshd(1, 100, 4, 128), bshd(1, 1500, 4, 128)
+    _assert_close(_run(q, k, is_causal=True), _oracle(q_cpu, k_cpu, is_causal=True), "strided causal")
+
+
 def test_deterministic_bits():
     q, k = _inputs((2, 8, 700, 64), (2, 8, 700, 64), seed=6)
     a = _run(q, k)
