@@ -217,17 +217,24 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     const uint32_t q_row_b = RAGGED ? (uint32_t)a.qs_s * 2u : (uint32_t)(D * 2), k_row_b = RAGGED ? (uint32_t)a.ks_s * 2u : (uint32_t)(D * 2);
     uint32_t q_voff[2] = {lrow * q_row_b + piece_b[0], lrow * q_row_b + piece_b[1]};
     uint32_t k_voff[2] = {lrow * k_row_b + piece_b[0], lrow * k_row_b + piece_b[1]};
-    const char *q_b = reinterpret_cast<const char *>(a.q + (int64_t)b * a.qs_b) + (int64_t)q0 * q_row_b;
-    const char *k_b = reinterpret_cast<const char *>(a.k + (int64_t)b * a.ks_b) + (int64_t)kbase * k_row_b;
+    // start of this batch entry's Q / K (head 0, row 0), and the same advanced to this wave's first
+    // row.  Only the whole-tile kernel addresses through the latter: there every row it names
+    // exists.  The ragged kernel and the rare slow path clamp ABSOLUTE row numbers instead, because
+    // a wave's rows (and whole tiles of them) may lie past the end of the tensor.
+    const char *q_batch = reinterpret_cast<const char *>(a.q + (int64_t)b * a.qs_b);
+    const char *k_batch = reinterpret_cast<const char *>(a.k + (int64_t)b * a.ks_b);
+    const int q_first = blk_row0 + qg * 32;  // this wave's first query row, unclamped
+    const char *q_b = q_batch + (int64_t)q0 * q_row_b;
+    const char *k_b = k_batch + (int64_t)min(kbase, a.Sk - 1) * k_row_b;
     const int64_t q_head_b = a.qs_h * 2, k_head_b = a.ks_h * 2;
     char *my_ring = ring + wave * (NS * SLOT_BYTES);
 
-    // DMA instruction `tt` (of NT) of a tile: rows [8*tt, 8*tt + 8) of the tile starting at `tile`
-    // (wave-uniform) go to ring slot `slot`.  In the ragged kernel a tile may run past the end of
-    // its tensor slice after `rows_left` rows; those rows are replaced by the last real row (the
-    // consumer masks or ignores them).  No branch either way: a taken branch costs a wave far
-    // more than the few address instructions it would skip.
-    auto fetch_piece = [&](const char *tile, uint32_t row_b, uint32_t (&voff)[2], int rows_left, int slot, int tt) {
+    // DMA instruction `tt` (of NT) of a tile: its rows [8*tt, 8*tt + 8) go to ring slot `slot`.
+    // Whole-tile kernel: `tile` (wave-uniform) is the tile's first row.  Ragged kernel: `tile` is
+    // row 0 of the head's slice, the tile starts at row `first_row` of its `n_rows`, and rows past
+    // the end are replaced by the last real row (the consumer masks or ignores them).  No branch
+    // either way: a taken branch costs a wave far more than the few address instructions it would skip.
+    auto fetch_piece = [&](const char *tile, uint32_t row_b, uint32_t (&voff)[2], int first_row, int n_rows, int slot, int tt) {
         char *dst = my_ring + slot * SLOT_BYTES;
         if (!RAGGED) {
             // every tile is whole and its rows are dense: instruction tt reads 1 KB further in
@@ -243,8 +250,8 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         } else {
             FCS_OPAQUE_V(lrow);
             FCS_OPAQUE_V(piece_b[tt & 1]);
-            const uint32_t row = (uint32_t)max(0, min(tt * 8 + lrow, rows_left - 1));
-            FCS_GLDS16(tile + (row * row_b + piece_b[tt & 1]), dst + tt * 1024);
+            const uint32_t row = (uint32_t)min(first_row + tt * 8 + lrow, n_rows - 1);
+            FCS_GLDS16(tile + ((size_t)row * row_b + piece_b[tt & 1]), dst + tt * 1024);
         }
     };
     // Read a ring slot back as an MFMA operand: lane (n, g) takes, for step tt, piece 2*tt + g of
@@ -314,10 +321,11 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 }
             }
         } else if (j == 0)
-            fetch_piece(q_b + (int64_t)hh * q_head_b, q_row_b, q_voff, a.Sq - q0, slot, tt);
+            fetch_piece((RAGGED ? q_batch : q_b) + (int64_t)hh * q_head_b, q_row_b, q_voff, q_first, a.Sq, slot, tt);
+        else if (RAGGED)
+            fetch_piece(k_batch + (int64_t)hh * k_head_b, k_row_b, k_voff, kbase + (j - 1) * 32, a.Sk, slot, tt);
         else
-            fetch_piece(k_b + (int64_t)hh * k_head_b + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff,
-                        a.Sk - kbase - (j - 1) * 32, slot, tt);
+            fetch_piece(k_b + (int64_t)hh * k_head_b + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff, 0, 0, slot, tt);
     };
     auto fetch_pos = [&](int h_now, int j_ahead, int slot) {
 #pragma unroll
@@ -467,9 +475,9 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             int lane_s = lane;
             FCS_OPAQUE_V(lane_s);
             const int n_s = lane_s & 31, g_s = lane_s >> 5;
-            const _Float16 *qp = reinterpret_cast<const _Float16 *>(q_b + (int64_t)h * q_head_b) +
-                                 (int64_t)min(n_s, a.Sq - 1 - q0) * a.qs_s + g_s * 8;
-            const _Float16 *kp = reinterpret_cast<const _Float16 *>(k_b + (int64_t)h * k_head_b) + g_s * 8;
+            const _Float16 *qp = reinterpret_cast<const _Float16 *>(q_batch + (int64_t)h * q_head_b) +
+                                 (int64_t)min(q_first + n_s, a.Sq - 1) * a.qs_s + g_s * 8;
+            const _Float16 *kp = reinterpret_cast<const _Float16 *>(k_batch + (int64_t)h * k_head_b) + g_s * 8;
             half8 qs[NT];
 #pragma unroll
             for (int tt = 0; tt < NT; ++tt) {
@@ -478,7 +486,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             }
             auto score_tile = [&](int t) {
                 half8 ks[NT];
-                const int krow = max(0, min(t * 32 + n_s, a.Sk - 1 - kbase));
+                const int krow = min(kbase + t * 32 + n_s, a.Sk - 1);
 #pragma unroll
                 for (int tt = 0; tt < NT; ++tt) ks[tt] = load8(kp + (int64_t)krow * a.ks_s + tt * 16);
                 floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
