@@ -217,6 +217,11 @@ def test_reference_error_handling():
     ((36, 1, 950, 64), (36, 1, 950, 64), {}),            # ... with an odd number of query blocks
     ((8, 2, 2048, 64), (8, 2, 2048, 64), {}),            # whole tiles, more workgroups than compute units
     ((40, 2, 96, 64), (40, 2, 96, 64), {"cls_len": 5}),  # waves whose rows all lie past the tensor
+    # key counts for which whole tiles, or a whole wave's range, start past the last key
+    ((4, 4, 917, 64), (4, 4, 917, 64), {}),
+    ((2, 1, 1310, 64), (2, 1, 1310, 64), {"cls_len": 5}),
+    ((2, 3, 1050, 64), (2, 3, 1050, 64), {"scale": 30.0}),
+    ((1, 2, 1550, 64), (1, 2, 1550, 64), {}),
     # few averaged rows (matrix-vector path): every row count, both head dims, ragged key counts,
     # several heads per workgroup, the largest score block it takes and the first it does not
     ((3, 5, 577, 64), (3, 5, 577, 64), {"cls_len": 2}),
