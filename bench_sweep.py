@@ -7,6 +7,9 @@ Counterpart of the reference's three sweeps (reference: benchmarks/benchmark_col
   noncausal           B = 1, H = 16, D = 64, S in {2048, ..., 262144}
   causal              B = 1, H = 32, Q_len = 128, D = 128, K_len in {16384, ..., 262144}
 
+plus one of this repository's own: `vit`, non-causal token counts of common vision encoders
+(197, 257, 577, 729, 1025, 1370), none of them a multiple of the kernels' 32-key tile.
+
 Timing follows the reference's `measure_latency` (benchmark_colsum.py:42-56): warm-up calls,
 then `iters` x (call + device synchronize) under one wall clock, so launch and host overhead
 are included.  Peak memory is `torch.cuda.max_memory_allocated` around one call
@@ -29,6 +32,9 @@ SWEEPS = {
     "noncausal_batched": [dict(B=b, H=16, Sq=1024, Sk=1024, D=64, causal=False) for b in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024)],
     "noncausal": [dict(B=1, H=16, Sq=s, Sk=s, D=64, causal=False) for s in (2048, 4096, 8192, 16384, 32768, 65536, 131072, 262144)],
     "causal": [dict(B=1, H=32, Sq=128, Sk=k, D=128, causal=True) for k in (16384, 32768, 65536, 131072, 262144)],
+    # not in the reference: token counts of common vision encoders (n*n patches + 1 class token)
+    "vit": [dict(B=b, H=h, Sq=s, Sk=s, D=64, causal=False) for (b, h, s) in
+            ((64, 12, 197), (32, 16, 257), (32, 16, 577), (16, 16, 729), (16, 16, 1025), (8, 16, 1370))],
 }
 EAGER_MAX_BYTES = 40 << 30  # logits + fp32 softmax + cast of the eager baseline must fit well inside HBM
 

@@ -215,6 +215,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     for (int par = 0; par < 2; ++par) piece_b[par] = (uint32_t)(((lane & 7) ^ ((par * 4 + (lane >> 4)) & 7)) * 16);
     // row pitch in bytes; a compile-time constant in the non-ragged kernel (rows are dense there)
     const uint32_t q_row_b = RAGGED ? (uint32_t)a.qs_s * 2u : (uint32_t)(D * 2), k_row_b = RAGGED ? (uint32_t)a.ks_s * 2u : (uint32_t)(D * 2);
+    uint32_t dense_voff[2] = {lrow * (uint32_t)(D * 2) + piece_b[0], lrow * (uint32_t)(D * 2) + piece_b[1]};  // ragged kernel's whole tiles
     uint32_t q_voff[2] = {lrow * q_row_b + piece_b[0], lrow * q_row_b + piece_b[1]};
     uint32_t k_voff[2] = {lrow * k_row_b + piece_b[0], lrow * k_row_b + piece_b[1]};
     // start of this batch entry's Q / K (head 0, row 0), and the same advanced to this wave's first
@@ -234,9 +235,10 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // row 0 of the head's slice, the tile starts at row `first_row` of its `n_rows`, and rows past
     // the end are replaced by the last real row (the consumer masks or ignores them).  No branch
     // either way: a taken branch costs a wave far more than the few address instructions it would skip.
-    auto fetch_piece = [&](const char *tile, uint32_t row_b, uint32_t (&voff)[2], int first_row, int n_rows, int slot, int tt) {
+    auto fetch_piece = [&](bool whole_tile, const char *tile, uint32_t row_b, uint32_t (&voff)[2], int first_row, int n_rows,
+                           int slot, int tt) {
         char *dst = my_ring + slot * SLOT_BYTES;
-        if (!RAGGED) {
+        if (whole_tile) {
             // every tile is whole and its rows are dense: instruction tt reads 1 KB further in
             // memory and writes 1 KB further in the slot, which is exactly what the immediate
             // offset does; base pointer, lane offset and LDS base are shared by the four pieces
@@ -321,15 +323,33 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 }
             }
         } else if (j == 0)
-            fetch_piece((RAGGED ? q_batch : q_b) + (int64_t)hh * q_head_b, q_row_b, q_voff, q_first, a.Sq, slot, tt);
-        else if (RAGGED)
-            fetch_piece(k_batch + (int64_t)hh * k_head_b, k_row_b, k_voff, kbase + (j - 1) * 32, a.Sk, slot, tt);
+            fetch_piece(true, q_b + (int64_t)hh * q_head_b, q_row_b, q_voff, 0, 0, slot, tt);
         else
-            fetch_piece(k_b + (int64_t)hh * k_head_b + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff, 0, 0, slot, tt);
+            fetch_piece(true, k_b + (int64_t)hh * k_head_b + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff, 0, 0, slot, tt);
     };
     auto fetch_pos = [&](int h_now, int j_ahead, int slot) {
+        if (RAGGED) {
+            // One wave-uniform decision per tile: a tile that lies wholly inside its tensor and has
+            // dense rows takes the cheap whole-tile form; only tiles that touch the end (or strided
+            // rows) pay for per-lane row clamping.
+            const int hh = min(h_now + j_ahead / ITEMS, h_end - 1);
+            const int j = j_ahead % ITEMS;
+            const bool is_q = (j == 0);
+            const char *slice = is_q ? q_batch + (int64_t)hh * q_head_b : k_batch + (int64_t)hh * k_head_b;
+            const int first_row = is_q ? q_first : kbase + (j - 1) * 32, n_rows = is_q ? a.Sq : a.Sk;
+            const uint32_t row_b = is_q ? q_row_b : k_row_b;
+            if (first_row + 32 <= n_rows && row_b == (uint32_t)(D * 2)) {
+                const char *tile = slice + (size_t)first_row * (D * 2);
 #pragma unroll
-        for (int tt = 0; tt < NT; ++tt) fetch_pos_piece(h_now, j_ahead, slot, tt);
+                for (int tt = 0; tt < NT; ++tt) fetch_piece(true, tile, row_b, dense_voff, 0, 0, slot, tt);
+            } else {
+#pragma unroll
+                for (int tt = 0; tt < NT; ++tt) fetch_piece(false, slice, row_b, dense_voff, first_row, n_rows, slot, tt);
+            }
+        } else {
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) fetch_pos_piece(h_now, j_ahead, slot, tt);
+        }
     };
     int sq = 0;  // ring slot of the current head's Q tile (only used when the slots are not static)
     auto slot_of = [&](int j) {  // slot of item j of the current head, j compile-time, j < ITEMS + 3
@@ -395,10 +415,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 
         // e = 2^(c*s) for tile t, in place, and its contribution to the row sums
         auto exp_tile = [&](int t) {
-            const bool real = !RAGGED || (kbase + t * 32 + n) < a.Sk;
+            // ragged: a key past the end gets the bias -inf, so its exponential is 0; the bias rides
+            // on the scale multiply (one FMA) instead of costing a select per score
+            const float bias = (!RAGGED || (kbase + t * 32 + n) < a.Sk) ? 0.f : -INFINITY;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const float e = real ? fast_exp2(PRE ? acc[t][i] : acc[t][i] * a.c) : 0.f;
+                const float e = fast_exp2(PRE ? acc[t][i] : (RAGGED ? fmaf(acc[t][i], a.c, bias) : acc[t][i] * a.c));
                 acc[t][i] = e;
                 rs[i] += e;
             }
