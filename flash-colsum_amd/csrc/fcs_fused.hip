@@ -160,7 +160,6 @@ template <int D, int TPW, bool RAGGED, int PRE, bool BF>
 __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 {
     static_assert(D == 64, "the fused path is laid out for 64-wide heads");
-    static_assert(!(PRE && RAGGED), "the pre-scaled variant needs whole tiles and dense rows");
     static_assert(!(PRE && BF), "the pre-scaled variant rounds Q*c to fp16; bf16 would be too coarse");
     constexpr int NT = D / 16;             // MFMA steps (and 16-byte pieces per lane) per operand tile
     constexpr int NS = 3;                  // ring slots per wave
@@ -313,13 +312,22 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         const int j = j_ahead % ITEMS;
         if (j == 0 && PRE) {
             if (tt == 0) {
-                const char *src = q_b + (int64_t)hh * q_head_b;
+                // whole-tile kernel: the wave's rows are one contiguous run; ragged kernel: row by row,
+                // clamped to the last real row (rows past the end carry weight 0)
+                const char *src;
+                if (RAGGED) {
+                    const int row_in_tile = (PRE == 8) ? kg * 4 + (lane >> 4) : kg * 8 + (lane >> 3);
+                    const int in_row_b = (PRE == 8) ? (lane & 15) * 8 : (lane & 7) * 16;
+                    src = q_batch + (int64_t)hh * q_head_b + (size_t)min(q_first + row_in_tile, a.Sq - 1) * q_row_b + in_row_b;
+                } else {
+                    src = q_b + (int64_t)hh * q_head_b + ((PRE == 8) ? kg * 512 + lane * 8 : kg * 1024 + lane * 16);
+                }
                 if (PRE == 8) {
-                    const uint2 v = *reinterpret_cast<const uint2 *>(src + kg * 512 + lane * 8);
+                    const uint2 v = *reinterpret_cast<const uint2 *>(src);
                     qraw[0] = v.x;
                     qraw[1] = v.y;
                 } else {
-                    qraw = *reinterpret_cast<const uint4v *>(src + kg * 1024 + lane * 16);
+                    qraw = *reinterpret_cast<const uint4v *>(src);
                 }
             }
         } else if (j == 0)
@@ -335,6 +343,10 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             const int hh = min(h_now + j_ahead / ITEMS, h_end - 1);
             const int j = j_ahead % ITEMS;
             const bool is_q = (j == 0);
+            if (PRE && is_q) {  // the Q item of the pre-scaled variant is a plain load, not a tile
+                fetch_pos_piece(h_now, j_ahead, slot, 0);
+                return;
+            }
             const char *slice = is_q ? q_batch + (int64_t)hh * q_head_b : k_batch + (int64_t)hh * k_head_b;
             const int first_row = is_q ? q_first : kbase + (j - 1) * 32, n_rows = is_q ? a.Sq : a.Sk;
             const uint32_t row_b = is_q ? q_row_b : k_row_b;
@@ -418,11 +430,22 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             // ragged: a key past the end gets the bias -inf, so its exponential is 0; the bias rides
             // on the scale multiply (one FMA) instead of costing a select per score
             const float bias = (!RAGGED || (kbase + t * 32 + n) < a.Sk) ? 0.f : -INFINITY;
+            if (PRE && RAGGED && kbase + t * 32 + 31 >= a.Sk) {
+                // pre-scaled scores have no multiply to carry the bias: only a tile that reaches
+                // past the last key (wave-uniform test) pays an add per score
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float e = fast_exp2(PRE ? acc[t][i] : (RAGGED ? fmaf(acc[t][i], a.c, bias) : acc[t][i] * a.c));
-                acc[t][i] = e;
-                rs[i] += e;
+                for (int i = 0; i < 16; ++i) {
+                    const float e = fast_exp2(acc[t][i] + bias);
+                    acc[t][i] = e;
+                    rs[i] += e;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float e = fast_exp2(PRE ? acc[t][i] : (RAGGED ? fmaf(acc[t][i], a.c, bias) : acc[t][i] * a.c));
+                    acc[t][i] = e;
+                    rs[i] += e;
+                }
             }
             // pinned here: otherwise the optimiser sinks every exponent below the last MFMA
             asm volatile("" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]), "+v"(rs[4]), "+v"(rs[5]), "+v"(rs[6]),
@@ -583,11 +606,16 @@ static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.f_nqblk * p.B, p.f_hg);  // x = batch entry * f_nqblk + row block
     const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
-    const bool pre = !BF && TPW == 8 && whole && (long)p.H * p.q_rows >= 4096 && fabsf(a.c) <= 0.1251f * 1.44269504f;
-    if (pre && p.f_kg == 8)
+    const bool pre = !BF && TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4) && (long)p.H * p.q_rows >= 4096 &&
+                     fabsf(a.c) <= 0.1251f * 1.44269504f;
+    if (pre && whole && TPW == 8 && p.f_kg == 8)
         hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 8, false>), grid, dim3(512), 0, st, a);
-    else if (pre && p.f_kg == 4)
+    else if (pre && whole && TPW == 8 && p.f_kg == 4)
         hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 4, false>), grid, dim3(512), 0, st, a);
+    else if (pre && p.f_kg == 8)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, (TPW >= 5 ? TPW : 8), true, 8, false>), grid, dim3(512), 0, st, a);
+    else if (pre)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, (TPW >= 5 ? TPW : 8), true, 4, false>), grid, dim3(512), 0, st, a);
     else if (whole)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false, 0, BF>), grid, dim3(512), 0, st, a);
     else

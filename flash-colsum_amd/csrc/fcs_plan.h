@@ -142,11 +142,24 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         p.f_qg = 8 / p.f_kg;
         p.f_tpw = ceil_div(tiles, p.f_kg);
         p.f_nqblk = ceil_div(p.q_rows, 32 * p.f_qg);
+        // Heads per workgroup: one workgroup is resident per compute unit, so the launch runs in
+        // generations of kComputeUnits workgroups, each as long as its heads plus about 0.6 of a
+        // head for starting and finishing.  Fewer heads per workgroup fill the last generation
+        // better (528 workgroups of 16 heads take three generations, 2112 of 4 take nine quarter-
+        // length ones) at the price of more starts and more partial slabs.
         const long basef = (long)p.f_nqblk * B;
-        int hg = (int)((512 + basef - 1) / basef);
-        if (hg > H) hg = H;
-        if (hg < 1) hg = 1;
-        p.f_hpg = ceil_div(H, hg);
+        double best = 0.;
+        p.f_hpg = H;
+        for (int hpg = H; hpg >= 1; --hpg) {
+            const int hg = ceil_div(H, hpg);
+            if (ceil_div(H, hg) != hpg) continue;  // same grouping as a smaller hpg
+            const long gens = (basef * hg + kComputeUnits - 1) / kComputeUnits;
+            const double cost = (double)gens * (hpg + 0.6) + 0.01 * hg;
+            if (hpg == H || cost < best) {
+                best = cost;
+                p.f_hpg = hpg;
+            }
+        }
         p.f_hg = ceil_div(H, p.f_hpg);
         p.n_partials = p.f_hg * p.f_nqblk * p.f_qg;
         size_t off = align256(sizeof(float) * (size_t)p.n_partials * B * Sk);

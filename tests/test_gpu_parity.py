@@ -251,6 +251,15 @@ def test_edge_shapes(qs, ks, kw):
     ((2, 4, 1024, 64), True, {"scale": -0.125}, 0.0),
     ((1, 8, 1024, 64), False, {}, 6.0),
     ((3, 4, 1024, 64), True, {}, 40.0),
+    # the same variant of the ragged kernel: token counts that are not a multiple of the tile
+    ((2, 8, 577, 64), False, {}, 0.0),
+    ((2, 8, 577, 64), True, {"scale": -0.125}, 0.0),
+    ((1, 4, 1025, 64), False, {}, 0.0),
+    ((1, 4, 1370, 64), True, {}, 0.0),
+    ((1, 3, 1536, 64), False, {"scale": 0.1}, 0.0),      # whole tiles, six per wave
+    ((2, 8, 577, 64), False, {}, 6.0),
+    ((1, 4, 1370, 64), True, {}, 40.0),
+    ((2, 8, 700, 64), False, {"cls_len": 600}, 0.0),
 ])
 def test_prescaled_shared_q_variant(shape, same, kw, boost):
     """Whole-tile S = 2048 or 1024, D = 64 launches with >= 4096 averaged (head, row) pairs and
