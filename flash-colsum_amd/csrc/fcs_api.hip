@@ -25,7 +25,6 @@ int run(int bf16, int causal, const void *q, const void *k, float *out, void *ou
 {
     if (!q || !k || !out || !qs || !ks) return FCS_E_NULL;
     if (B < 1 || H < 1 || Sq < 1 || Sk < 1 || D < 1 || cls_n == 0 || k_past < 0) return FCS_E_DIMS;
-    if ((long)B * H > 65535) return FCS_E_DIMS;
     if (D != 64 && D != 128) return FCS_E_HEAD_DIM;
     if (!strides_ok(qs, B > 1) || !strides_ok(ks, B > 1) || !aligned16(q) || !aligned16(k)) return FCS_E_STRIDE;
     if (!isfinite(scale)) return FCS_E_SCALE;
@@ -33,6 +32,9 @@ int run(int bf16, int causal, const void *q, const void *k, float *out, void *ou
     fcs::Plan p;
     if (!fcs::make_plan(p, causal, B, H, Sq, Sk, D, cls_n, k_past)) return FCS_E_DIMS;
     p.bf16 = bf16;
+    // only the two-pass kernels put (batch entry, head) on a 16-bit grid axis
+    if (!p.fused && !p.fewrows && (long)B * H > 65535) return FCS_E_DIMS;
+    if (ws && (reinterpret_cast<uintptr_t>(ws) & 255u)) return FCS_E_WORKSPACE;
     if (p.total > 0 && (!ws || ws_bytes < p.total)) return ws ? FCS_E_WORKSPACE : FCS_E_NULL;
 
     fcs::Args a;
@@ -72,10 +74,10 @@ const char *fcs_strerror(int code)
     switch (code) {
     case FCS_OK: return "ok";
     case FCS_E_NULL: return "a required pointer is NULL";
-    case FCS_E_DIMS: return "invalid dimension (each of B,H,S,D must be >= 1, B*H <= 65535, cls_n != 0, k_past >= 0)";
+    case FCS_E_DIMS: return "invalid dimension (each of B,H,S,D must be >= 1, cls_n != 0, k_past >= 0; B*H <= 65535 on the two-pass path)";
     case FCS_E_HEAD_DIM: return "unsupported head dim (compiled: 64, 128)";
     case FCS_E_STRIDE: return "unsupported layout (last stride must be 1; rows, heads and base 16-byte aligned)";
-    case FCS_E_WORKSPACE: return "workspace smaller than fcs_workspace_bytes()";
+    case FCS_E_WORKSPACE: return "workspace smaller than fcs_workspace_bytes() or not 256-byte aligned";
     case FCS_E_SCALE: return "scale is not finite";
     default: return code > 0 ? "HIP launch error (code is a hipError_t)" : "unknown error code";
     }

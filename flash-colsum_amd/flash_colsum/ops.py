@@ -17,7 +17,7 @@ def _validated(query, key, scale, is_causal, cls_len):
     if query.ndim != 4 or key.ndim != 4:
         raise ValueError(f"Expected 4D tensors, got query.ndim={query.ndim}, key.ndim={key.ndim}")
     if query.device.type != "cuda":
-        raise ValueError(f"flash_colsum only supports CUDA (HIP) tensors, got {query.device}")
+        raise ValueError(f"Flash attention only supports CUDA tensors, got {query.device}")
     if cls_len is not None:
         if is_causal:
             raise ValueError("cls_len is only supported for non-causal attention")

@@ -1,0 +1,63 @@
+"""The entry point that allocates nothing: fcs_colsum_noncausal_f16_static keeps its partial
+column-sum slabs in a static per-GPU device array instead of a caller workspace.  It must give
+the bits of fcs_colsum_noncausal_f16 (same kernels, same launch plan) on two calls in a row, the
+second with a smaller input that leaves stale slabs of the first behind in the array."""
+import ctypes
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _call(lib, static, q, k, cls_n, scale):
+    b, h, s, d = q.shape
+    out = torch.full((b, s), float("nan"), dtype=torch.float32, device="cuda")
+    out_h = torch.full((b, s), float("nan"), dtype=torch.float16, device="cuda")
+    qs, ks = (ctypes.c_int64 * 4)(*q.stride()), (ctypes.c_int64 * 4)(*k.stride())
+    stream = torch.cuda.current_stream().cuda_stream
+    if static:
+        rc = lib.fcs_colsum_noncausal_f16_static(q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h.data_ptr(),
+                                                 b, h, s, d, qs, ks, scale, cls_n, stream)
+    else:
+        n_ws = lib.fcs_workspace_bytes(0, b, h, s, s, d, cls_n)
+        ws = torch.empty(max(n_ws, 1), dtype=torch.uint8, device="cuda")
+        rc = lib.fcs_colsum_noncausal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h.data_ptr(), ws.data_ptr(),
+                                          n_ws, b, h, s, d, qs, ks, scale, cls_n, stream)
+    torch.cuda.synchronize()
+    return rc, out, out_h
+
+
+def test_static_scratch_entry_point_matches_the_workspace_one():
+    from flash_colsum import _hip
+    from oracle import colsum_exact
+
+    lib = _hip.lib()
+    g = torch.Generator().manual_seed(31)
+    # larger call first (fused path, 4 MiB of slabs), then smaller ones that reuse the dirty array:
+    # a ragged fused call, a two-pass call (row statistics + partials) and a few-rows call
+    cases = [((8, 16, 2048, 64), -1, 0.125), ((3, 5, 333, 64), -1, 0.2), ((2, 3, 300, 128), -1, 0.1),
+             ((4, 6, 577, 64), 1, 0.125), ((1, 2, 40, 64), -1, 0.125)]
+    for shape, cls_n, scale in cases:
+        q = torch.randn(shape, generator=g).half()
+        k = torch.randn(shape, generator=g).half()
+        qc, kc = q.cuda(), k.cuda()
+        print("static entry point", shape, cls_n, flush=True)
+        rc0, want, want_h = _call(lib, False, qc, kc, cls_n, scale)
+        rc1, got, got_h = _call(lib, True, qc, kc, cls_n, scale)
+        assert rc0 == 0 and rc1 == 0, (shape, rc0, rc1)
+        assert torch.equal(got, want) and torch.equal(got_h, want_h), shape
+        ref = colsum_exact(q, k, scale=scale, cls_len=None if cls_n < 0 else cls_n)
+        err = (got.cpu().double() - ref).abs()
+        assert err.max().item() <= 1e-4 and (err / ref.abs().clamp_min(1e-9)).max().item() <= 1e-3, shape
+
+
+def test_static_scratch_entry_point_rejects_what_does_not_fit():
+    from flash_colsum import _hip
+
+    lib = _hip.lib()
+    p = ctypes.c_void_p(4096)  # never dereferenced
+    st = (ctypes.c_int64 * 4)(64 * 16 * 2048 * 64, 2048 * 64, 64, 1)
+    assert lib.fcs_workspace_bytes(0, 64, 16, 2048, 2048, 64, -1) > (8 << 20)
+    assert lib.fcs_colsum_noncausal_f16_static(p, p, p, None, 64, 16, 2048, 64, st, st, 0.125, -1, None) == -7
+    assert "static scratch" in _hip.strerror(-7)
