@@ -3,10 +3,39 @@
 #include <math.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "flash_colsum.h"
 #include "fcs_kernels.h"
 
+// Workspace of fcs_colsum_noncausal_f16_static(): one copy per GPU, held until the process ends.
+// Host code never uses this name as an address (it is only a handle for hipGetSymbolAddress).
+static __device__ __align__(256) unsigned char fcs_static_scratch[FCS_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];  // device address of fcs_static_scratch on each GPU, looked up once
+std::once_flag g_scratch_once[kMaxDevices];
+hipError_t g_scratch_err[kMaxDevices];
+
+// Device address of the current GPU's copy of the static scratch array; no allocation.
+hipError_t static_scratch(void **ptr)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::call_once(g_scratch_once[dev], [dev]() {
+        void *p = nullptr;
+        g_scratch_err[dev] = hipGetSymbolAddress(&p, HIP_SYMBOL(fcs_static_scratch));
+        g_scratch_ptr[dev] = (g_scratch_err[dev] == hipSuccess) ? p : nullptr;
+    });
+    if (g_scratch_err[dev] != hipSuccess) return g_scratch_err[dev];
+    if (!g_scratch_ptr[dev]) return hipErrorInvalidSymbol;
+    *ptr = g_scratch_ptr[dev];
+    return hipSuccess;
+}
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -78,6 +107,7 @@ const char *fcs_strerror(int code)
     case FCS_E_HEAD_DIM: return "unsupported head dim (compiled: 64, 128)";
     case FCS_E_STRIDE: return "unsupported layout (last stride must be 1; rows, heads and base 16-byte aligned)";
     case FCS_E_WORKSPACE: return "workspace smaller than fcs_workspace_bytes() or not 256-byte aligned";
+    case FCS_E_STATIC_LIMIT: return "the call needs more workspace than the static scratch holds (FCS_STATIC_SCRATCH_BYTES)";
     case FCS_E_SCALE: return "scale is not finite";
     default: return code > 0 ? "HIP launch error (code is a hipError_t)" : "unknown error code";
     }
@@ -97,6 +127,22 @@ int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *out
 {
     return run(0, 0, q, k, out, out_f16, ws, ws_bytes, B, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
                hip_stream);
+}
+
+int fcs_colsum_noncausal_f16_static(const void *q, const void *k, float *out, void *out_f16, int B, int H, int S, int D,
+                                    const int64_t q_strides[4], const int64_t k_strides[4], float scale, int cls_n,
+                                    void *hip_stream)
+{
+    // size check first: it needs no GPU, like every other argument error
+    fcs::Plan p;
+    if (!fcs::make_plan(p, 0, B, H, S, S, D, cls_n < 0 ? -1 : cls_n, 0)) return FCS_E_DIMS;
+    if (p.total > (size_t)FCS_STATIC_SCRATCH_BYTES) return FCS_E_STATIC_LIMIT;
+    if (!q || !k || !out || !q_strides || !k_strides) return FCS_E_NULL;
+    void *ws = nullptr;
+    const hipError_t e = static_scratch(&ws);
+    if (e != hipSuccess) return (int)e;
+    return run(0, 0, q, k, out, out_f16, ws, FCS_STATIC_SCRATCH_BYTES, B, H, S, S, D, q_strides, k_strides, scale,
+               cls_n < 0 ? -1 : cls_n, 0, hip_stream);
 }
 
 int fcs_colsum_noncausal_bf16(const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes, int B, int H,

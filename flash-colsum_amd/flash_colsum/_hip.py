@@ -16,7 +16,7 @@ from typing import Optional
 import torch
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libflashcolsum.so")
-_ABI_VERSION = 3
+_ABI_VERSION = 4
 _lib = None
 
 _I64x4 = ctypes.c_int64 * 4
@@ -46,6 +46,12 @@ def lib() -> ctypes.CDLL:
                 ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                 ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
                 ctypes.c_float, ctypes.c_int, ctypes.c_void_p]
+        cdll.fcs_colsum_noncausal_f16_static.restype = ctypes.c_int
+        cdll.fcs_colsum_noncausal_f16_static.argtypes = [
+            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+            ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+            ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
+            ctypes.c_float, ctypes.c_int, ctypes.c_void_p]
         for fn in (cdll.fcs_colsum_causal_f16, cdll.fcs_colsum_causal_bf16):
             fn.restype = ctypes.c_int
             fn.argtypes = [

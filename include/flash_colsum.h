@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FCS_ABI_VERSION 3
+#define FCS_ABI_VERSION 4
 
 enum {
     FCS_OK = 0,
@@ -35,8 +35,13 @@ enum {
     FCS_E_STRIDE = -4,    /* last-dim stride != 1, or a stride / base not 16-B aligned   */
     FCS_E_WORKSPACE = -5, /* ws_bytes smaller than fcs_workspace_bytes() for these dims,
                              or ws not 256-byte aligned                                  */
-    FCS_E_SCALE = -6      /* scale is NaN or infinite                                    */
+    FCS_E_SCALE = -6,     /* scale is NaN or infinite                                    */
+    FCS_E_STATIC_LIMIT = -7 /* fcs_colsum_noncausal_f16_static: the call needs more workspace
+                               than FCS_STATIC_SCRATCH_BYTES                               */
 };
+
+/* Size of the per-GPU static scratch array behind fcs_colsum_noncausal_f16_static(). */
+#define FCS_STATIC_SCRATCH_BYTES (8u << 20)
 
 /* ABI version of the loaded library (== FCS_ABI_VERSION of the header it was built with). */
 int fcs_abi_version(void);
@@ -70,6 +75,20 @@ int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *out
                              int B, int H, int S, int D,
                              const int64_t q_strides[4], const int64_t k_strides[4],
                              float scale, int cls_n, void *hip_stream);
+
+/* fcs_colsum_noncausal_f16 for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): same arguments minus
+ * the workspace, which is a static device array of FCS_STATIC_SCRATCH_BYTES that every GPU
+ * the library runs on holds until the process ends.  Has no counterpart in the reference.
+ * Calls no hipMalloc / hipFree or any allocating routine.  Returns FCS_E_STATIC_LIMIT when
+ * fcs_workspace_bytes(0, B, H, S, S, D, cls_n) exceeds FCS_STATIC_SCRATCH_BYTES (8 MiB: enough
+ * for B=8 H=16 S=2048 D=64, which needs 4 MiB).  All calls on one GPU share that GPU's array:
+ * calls that overlap in time on one GPU (different streams or threads) race; calls on one
+ * stream are ordered and safe.  Results are bit-identical to fcs_colsum_noncausal_f16. */
+int fcs_colsum_noncausal_f16_static(const void *q, const void *k, float *out, void *out_f16,
+                                    int B, int H, int S, int D,
+                                    const int64_t q_strides[4], const int64_t k_strides[4],
+                                    float scale, int cls_n, void *hip_stream);
 
 /* Causal column means for one sequence (batch 1), fp16 inputs, fp32 output.
  *   q          (1,H,Q_len,D), k (1,H,K_len,D) fp16; strides as above (index 0 ignored).
