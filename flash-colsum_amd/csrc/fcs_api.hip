@@ -48,12 +48,14 @@ bool strides_ok(const int64_t s[4], bool use_batch)
     return true;
 }
 
+// H = query heads, Hk = key heads (H % Hk == 0; query head h reads key head h / (H / Hk))
 int run(int bf16, int causal, const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes, int B, int H,
-        int Sq, int Sk, int D, const int64_t qs[4], const int64_t ks[4], float scale, int cls_n,
+        int Hk, int Sq, int Sk, int D, const int64_t qs[4], const int64_t ks[4], float scale, int cls_n,
         int k_past, void *stream)
 {
     if (!q || !k || !out || !qs || !ks) return FCS_E_NULL;
-    if (B < 1 || H < 1 || Sq < 1 || Sk < 1 || D < 1 || cls_n == 0 || k_past < 0) return FCS_E_DIMS;
+    if (B < 1 || H < 1 || Hk < 1 || Sq < 1 || Sk < 1 || D < 1 || cls_n == 0 || k_past < 0) return FCS_E_DIMS;
+    if (H % Hk != 0) return FCS_E_DIMS;
     if (D != 64 && D != 128) return FCS_E_HEAD_DIM;
     if (!strides_ok(qs, B > 1) || !strides_ok(ks, B > 1) || !aligned16(q) || !aligned16(k)) return FCS_E_STRIDE;
     if (!isfinite(scale)) return FCS_E_SCALE;
@@ -73,13 +75,15 @@ int run(int bf16, int causal, const void *q, const void *k, float *out, void *ou
     a.qs_b = qs[0]; a.qs_h = qs[1]; a.qs_s = qs[2];
     a.ks_b = ks[0]; a.ks_h = ks[1]; a.ks_s = ks[2];
     a.B = B; a.H = H; a.Sq = Sq; a.Sk = Sk;
+    a.kv_group = H / Hk;
+    a.kv_magic = (uint32_t)((0x100000000ull + (uint64_t)a.kv_group - 1) / (uint64_t)a.kv_group);  // unused when the group is 1
     a.q_rows = p.q_rows;
     a.causal = p.causal; a.k_past = p.k_past;
     a.negate = scale < 0.f;
     a.c = fabsf(scale) * 1.44269504088896340736f;
     a.n_chunks = p.n_chunks; a.chunk_keys = p.chunk_keys; a.rows_pad = p.rows_pad;
     char *w = static_cast<char *>(ws);
-    a.lse = reinterpret_cast<float *>(w + p.off_lse);
+    a.lse = reinterpret_cast<float2 *>(w + p.off_lse);
     a.ml = reinterpret_cast<float2 *>(w + p.off_ml);
     a.gh = p.gh; a.gq = p.gq;
     a.heads_per_group = p.heads_per_group; a.qtiles_per_group = p.qtiles_per_group;
@@ -103,10 +107,11 @@ const char *fcs_strerror(int code)
     switch (code) {
     case FCS_OK: return "ok";
     case FCS_E_NULL: return "a required pointer is NULL";
-    case FCS_E_DIMS: return "invalid dimension (each of B,H,S,D must be >= 1, cls_n != 0, k_past >= 0; B*H <= 65535 on the two-pass path)";
+    case FCS_E_DIMS: return "invalid dimension (each of B,H,S,D must be >= 1, Hq a multiple of Hk, cls_n != 0, k_past >= 0; B*H <= 65535 on the two-pass path)";
     case FCS_E_HEAD_DIM: return "unsupported head dim (compiled: 64, 128)";
     case FCS_E_STRIDE: return "unsupported layout (last stride must be 1; rows, heads and base 16-byte aligned)";
     case FCS_E_WORKSPACE: return "workspace smaller than fcs_workspace_bytes() or not 256-byte aligned";
+    case FCS_E_DTYPE: return "unknown operand dtype (FCS_DTYPE_F16 or FCS_DTYPE_BF16)";
     case FCS_E_STATIC_LIMIT: return "the call needs more workspace than the static scratch holds (FCS_STATIC_SCRATCH_BYTES)";
     case FCS_E_SCALE: return "scale is not finite";
     default: return code > 0 ? "HIP launch error (code is a hipError_t)" : "unknown error code";
@@ -125,8 +130,17 @@ int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *out
                              int S, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
                              int cls_n, void *hip_stream)
 {
-    return run(0, 0, q, k, out, out_f16, ws, ws_bytes, B, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
+    return run(0, 0, q, k, out, out_f16, ws, ws_bytes, B, H, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
                hip_stream);
+}
+
+int fcs_colsum_general(int dtype, int causal, const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes,
+                       int B, int Hq, int Hk, int Sq, int Sk, int D, int cls_n, int k_past, const int64_t q_strides[4],
+                       const int64_t k_strides[4], float scale, void *hip_stream)
+{
+    if (dtype != FCS_DTYPE_F16 && dtype != FCS_DTYPE_BF16) return FCS_E_DTYPE;
+    return run(dtype == FCS_DTYPE_BF16, causal ? 1 : 0, q, k, out, out_f16, ws, ws_bytes, B, Hq, Hk, Sq, Sk, D, q_strides,
+               k_strides, scale, cls_n < 0 ? -1 : cls_n, causal ? k_past : 0, hip_stream);
 }
 
 int fcs_colsum_noncausal_f16_static(const void *q, const void *k, float *out, void *out_f16, int B, int H, int S, int D,
@@ -141,7 +155,7 @@ int fcs_colsum_noncausal_f16_static(const void *q, const void *k, float *out, vo
     void *ws = nullptr;
     const hipError_t e = static_scratch(&ws);
     if (e != hipSuccess) return (int)e;
-    return run(0, 0, q, k, out, out_f16, ws, FCS_STATIC_SCRATCH_BYTES, B, H, S, S, D, q_strides, k_strides, scale,
+    return run(0, 0, q, k, out, out_f16, ws, FCS_STATIC_SCRATCH_BYTES, B, H, H, S, S, D, q_strides, k_strides, scale,
                cls_n < 0 ? -1 : cls_n, 0, hip_stream);
 }
 
@@ -149,7 +163,7 @@ int fcs_colsum_noncausal_bf16(const void *q, const void *k, float *out, void *ou
                               int S, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
                               int cls_n, void *hip_stream)
 {
-    return run(1, 0, q, k, out, out_f16, ws, ws_bytes, B, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
+    return run(1, 0, q, k, out, out_f16, ws, ws_bytes, B, H, H, S, S, D, q_strides, k_strides, scale, cls_n < 0 ? -1 : cls_n, 0,
                hip_stream);
 }
 
@@ -157,7 +171,7 @@ int fcs_colsum_causal_f16(const void *q, const void *k, float *out, void *out_f1
                           int K_len, int D, int k_past, const int64_t q_strides[4], const int64_t k_strides[4],
                           float scale, void *hip_stream)
 {
-    return run(0, 1, q, k, out, out_f16, ws, ws_bytes, 1, H, Q_len, K_len, D, q_strides, k_strides, scale, -1, k_past,
+    return run(0, 1, q, k, out, out_f16, ws, ws_bytes, 1, H, H, Q_len, K_len, D, q_strides, k_strides, scale, -1, k_past,
                hip_stream);
 }
 
@@ -165,7 +179,7 @@ int fcs_colsum_causal_bf16(const void *q, const void *k, float *out, void *out_f
                            int K_len, int D, int k_past, const int64_t q_strides[4], const int64_t k_strides[4],
                            float scale, void *hip_stream)
 {
-    return run(1, 1, q, k, out, out_f16, ws, ws_bytes, 1, H, Q_len, K_len, D, q_strides, k_strides, scale, -1, k_past,
+    return run(1, 1, q, k, out, out_f16, ws, ws_bytes, 1, H, H, Q_len, K_len, D, q_strides, k_strides, scale, -1, k_past,
                hip_stream);
 }
 

@@ -37,6 +37,12 @@ __device__ __forceinline__ floatx16 mfma16(half8 a, half8 b, floatx16 c)
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 }
 
+// key head of query head h (grouped-query attention): h / group through a multiply-high
+__device__ __forceinline__ int kv_head(int h, int group, uint32_t magic)
+{
+    return group == 1 ? h : (int)__umulhi((uint32_t)h, magic);
+}
+
 // Row of a 32x32 MFMA result tile held by accumulator register i of a lane in half-wave g
 // (the column is lane % 32).
 __device__ __forceinline__ int acc_row(int i, int g) { return 8 * (i >> 2) + 4 * g + (i & 3); }

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void fcs_fewrows_kernel(const Args a)
     constexpr int RPW = 64 / LPR;  // key rows per wave per load instruction
     constexpr int RPB = 4 * RPW;   // key rows per block per round
     constexpr int UN = 8;          // rounds in flight
-    __shared__ float sc[kFewRowsMaxScores];  // [R][Sk] scores in log2 units, then exponentials
+    __shared__ float sc[kFewRowsMaxScores];  // [R][Sk] scores, then exponentials
     __shared__ float slot[4];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void fcs_fewrows_kernel(const Args a)
 
     for (int h = h_begin; h < h_end; ++h) {
         const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h + sub * 8;
-        const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)h * a.ks_h + sub * 8;
+        const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)kv_head(h, a.kv_group, a.kv_magic) * a.ks_h + sub * 8;
         half8 qv[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void fcs_fewrows_kernel(const Args a)
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const float s = row_lanes_sum<LPR>(dot8<BF>(qv[r], kv[u]));
-                    if (sub == 0 && row < Sk) sc[r * Sk + row] = s * a.c;
+                    if (sub == 0 && row < Sk) sc[r * Sk + row] = s;  // raw score: scaled after the maximum is subtracted
                 }
             }
         }
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256) void fcs_fewrows_kernel(const Args a)
             m = block_reduce<true>(m, slot, lane, wave);
             float l = 0.f;
             for (int j = tid; j < Sk; j += 256) {
-                const float e = fast_exp2(sc[r * Sk + j] - m);
+                const float e = fast_exp2((sc[r * Sk + j] - m) * a.c);
                 sc[r * Sk + j] = e;  // each thread re-reads only what it wrote
                 l += e;
             }

@@ -306,6 +306,16 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // them and publishes them in `qshare`.
     uint4v qraw = {0u, 0u, 0u, 0u};
     auto item_vm = [&](int j_ahead) { return (PRE && (j_ahead % ITEMS) == 0) ? 1 : NT; };  // VMEM instructions of an item
+    // byte offsets of the key heads of the current and of the next query head (grouped key heads:
+    // head / kv_group), refreshed once per head instead of at every fetch
+    constexpr int HEADS_AHEAD = (ITEMS + NS - 1) / ITEMS;  // the look-ahead reaches this many heads past the current one
+    int64_t k_off[HEADS_AHEAD + 1];
+    auto set_k_off = [&](int h_now) {
+#pragma unroll
+        for (int i = 0; i <= HEADS_AHEAD; ++i)
+            k_off[i] = (int64_t)kv_head(min(h_now + i, h_end - 1), a.kv_group, a.kv_magic) * k_head_b;
+    };
+    set_k_off(h_begin);
     auto fetch_pos_piece = [&](int h_now, int j_ahead /* item index counted from the Q tile of head h_now, compile-time */,
                                int slot, int tt) {
         const int hh = min(h_now + j_ahead / ITEMS, h_end - 1);
@@ -333,7 +343,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         } else if (j == 0)
             fetch_piece(true, q_b + (int64_t)hh * q_head_b, q_row_b, q_voff, 0, 0, slot, tt);
         else
-            fetch_piece(true, k_b + (int64_t)hh * k_head_b + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff, 0, 0, slot, tt);
+            fetch_piece(true, k_b + k_off[j_ahead / ITEMS] + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff, 0, 0, slot, tt);
     };
     auto fetch_pos = [&](int h_now, int j_ahead, int slot) {
         if (RAGGED) {
@@ -347,7 +357,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 fetch_pos_piece(h_now, j_ahead, slot, 0);
                 return;
             }
-            const char *slice = is_q ? q_batch + (int64_t)hh * q_head_b : k_batch + (int64_t)hh * k_head_b;
+            const char *slice = is_q ? q_batch + (int64_t)hh * q_head_b : k_batch + k_off[j_ahead / ITEMS];
             const int first_row = is_q ? q_first : kbase + (j - 1) * 32, n_rows = is_q ? a.Sq : a.Sk;
             const uint32_t row_b = is_q ? q_row_b : k_row_b;
             if (first_row + 32 <= n_rows && row_b == (uint32_t)(D * 2)) {
@@ -409,6 +419,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 
     for (int unit = 0; unit < n_units; ++unit) {
         const int h = h_begin + unit;
+        set_k_off(h);
         // this head's Q tile and first key tile (fetched during the previous head).  (Reading them
         // back earlier, under the previous head's column-sum FMAs, makes them live across the loop
         // and the kernel spills.)
@@ -522,7 +533,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             const int n_s = lane_s & 31, g_s = lane_s >> 5;
             const _Float16 *qp = reinterpret_cast<const _Float16 *>(q_batch + (int64_t)h * q_head_b) +
                                  (int64_t)min(q_first + n_s, a.Sq - 1) * a.qs_s + g_s * 8;
-            const _Float16 *kp = reinterpret_cast<const _Float16 *>(k_batch + (int64_t)h * k_head_b) + g_s * 8;
+            const _Float16 *kp = reinterpret_cast<const _Float16 *>(k_batch + (int64_t)kv_head(h, a.kv_group, a.kv_magic) * k_head_b) + g_s * 8;
             half8 qs[NT];
 #pragma unroll
             for (int tt = 0; tt < NT; ++tt) {
@@ -550,12 +561,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 for (int i = 0; i < 16; ++i) v16[i] = fmaxf(v16[i], real ? c[i] : kNegBig);
             }
             reduce_rows<true>(v16, rr, kg_n, qg, kg, lane_s, [&](int, float m) { return m; });
-            float nm[16];
+            float rmax[16];  // subtracted from the scores BEFORE the scale: exact for scores of any size
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const floatx4 m4 = row_values(rr, i4, g_s);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) nm[4 * i4 + j] = -m4[j] * a.c;
+                for (int j = 0; j < 4; ++j) rmax[4 * i4 + j] = m4[j];
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) v16[i] = 0.f;
@@ -564,7 +575,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 const floatx16 c = score_tile(t);
                 const bool real = (kbase + t * 32 + n_s) < a.Sk;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) v16[i] += real ? fast_exp2(fmaf(c[i], a.c, nm[i])) : 0.f;
+                for (int i = 0; i < 16; ++i) v16[i] += real ? fast_exp2((c[i] - rmax[i]) * a.c) : 0.f;
             }
             reduce_rows<false>(v16, rr, kg_n, qg, kg, lane_s, [&](int row, float L) {
                 return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
@@ -581,7 +592,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 const bool real = (kbase + t * 32 + n_s) < a.Sk;
                 float sum = 0.f;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) sum = fmaf(real ? fast_exp2(fmaf(c[i], a.c, nm[i])) : 0.f, v16[i], sum);
+                for (int i = 0; i < 16; ++i) sum = fmaf(real ? fast_exp2((c[i] - rmax[i]) * a.c) : 0.f, v16[i], sum);
 #pragma unroll
                 for (int u = 0; u < TPW; ++u)  // col_acc lives in registers: static index only
                     if (u == t) col_acc[u] += sum;

@@ -13,14 +13,17 @@ struct Args {
     int64_t qs_b, qs_h, qs_s;  // element strides (last dim is 1)
     int64_t ks_b, ks_h, ks_s;
     int B, H, Sq, Sk;
+    int kv_group;        // query heads per key head (1 unless grouped-query): key head = head / kv_group
+    uint32_t kv_magic;   // ceil(2^32 / kv_group), for the division above (unused when kv_group == 1)
     int q_rows;          // query rows that are averaged
     int causal, k_past;  // key j visible to query i  <=>  j <= k_past + i
     int negate;          // scale < 0: scores are negated by flipping the stationary operand's sign
     float c;             // |scale| * log2(e)
     // pass 1
     int n_chunks, chunk_keys, rows_pad;
-    float *lse;   // [B*H][rows_pad]
-    float2 *ml;   // [B*H][n_chunks][rows_pad]
+    float2 *lse;  // [B*H][rows_pad]            (m, log2 l): row maximum in score units (0 on the
+                  //                            unstabilised path) and log2 of sum_j 2^((s_ij - m) * c)
+    float2 *ml;   // [B*H][n_chunks][rows_pad]  (m, l) of each key split
     // pass 2
     int gh, gq, heads_per_group, qtiles_per_group;
     float *partial;  // [gh*gq][B][Sk]

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
     const int q0 = bx * (WAVES * QW);
     const int qw0 = q0 + wave * QW;
     const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
-    const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)h * a.ks_h;
+    const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)kv_head(h, a.kv_group, a.kv_magic) * a.ks_h;
 
     // key range of this block: its split, cut at the last key any of its rows may see
     const int kc0 = chunk * a.chunk_keys;
@@ -226,12 +226,11 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
                     for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, acc[na][nb][i]);
                 const float mn = fmaxf(m[nb], tmax);
                 const float alpha = fast_exp2((m[nb] - mn) * a.c);
-                const float nm = -mn * a.c;
-                float sum = 0.f;
+                float sum = 0.f;  // the maximum is subtracted BEFORE the scale: exact for scores of any size
 #pragma unroll
                 for (int na = 0; na < NA; ++na)
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) sum += fast_exp2(fmaf(acc[na][nb][i], a.c, nm));
+                    for (int i = 0; i < 16; ++i) sum += fast_exp2((acc[na][nb][i] - mn) * a.c);
                 l[nb] = l[nb] * alpha + sum;
                 m[nb] = mn;
             } else {
@@ -245,14 +244,13 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
                     }
                 const float mn = fmaxf(m[nb], tmax);
                 const float alpha = fast_exp2((m[nb] - mn) * a.c);
-                const float nm = -mn * a.c;
                 float sum = 0.f;
 #pragma unroll
                 for (int na = 0; na < NA; ++na)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const bool vis = (kb + na * 32 + acc_row(i, g)) <= thr[nb];
-                        const float e = fast_exp2(fmaf(acc[na][nb][i], a.c, nm));
+                        const float e = fast_exp2((acc[na][nb][i] - mn) * a.c);
                         sum += vis ? e : 0.f;
                     }
                 l[nb] = l[nb] * alpha + sum;
@@ -274,11 +272,14 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
         const float ll = l[nb] * fast_exp2((m[nb] - mm) * a.c) + l2 * fast_exp2((m2 - mm) * a.c);
         if (g == 0) {
             const int qi = qw0 + nb * 32 + r;  // < rows_pad by construction
+            // the maximum stays in score units and apart from log2 l: folding m * c into one fp32
+            // would round it at the magnitude of m * c, which the later 2^(...) cannot undo
+            float2 v;
+            v.x = mm;
             if (a.n_chunks == 1) {
-                a.lse[(int64_t)bh * a.rows_pad + qi] = mm * a.c + fast_log2(ll);
+                v.y = fast_log2(ll);
+                a.lse[(int64_t)bh * a.rows_pad + qi] = v;
             } else {
-                float2 v;
-                v.x = mm * a.c;
                 v.y = ll;
                 a.ml[((int64_t)bh * a.n_chunks + chunk) * a.rows_pad + qi] = v;
             }
@@ -286,7 +287,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
     }
 }
 
-// merge the per-split (max, sum) partials of pass 1 into lse2: one thread per row, eight partials
+// merge the per-split (max, sum) partials of pass 1 into (max, log2 sum): one thread per row, eight partials
 // loaded at a time and folded in split order (fixed order: bit-reproducible)
 __global__ __launch_bounds__(64) void fcs_merge_stats_kernel(const Args a)
 {
@@ -306,11 +307,14 @@ __global__ __launch_bounds__(64) void fcs_merge_stats_kernel(const Args a)
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const float mn = fmaxf(mm, v[j].x);
-            ll = ll * fast_exp2(mm - mn) + v[j].y * fast_exp2(v[j].x - mn);
+            ll = ll * fast_exp2((mm - mn) * a.c) + v[j].y * fast_exp2((v[j].x - mn) * a.c);
             mm = mn;
         }
     }
-    a.lse[(int64_t)bh * a.rows_pad + i] = mm + fast_log2(ll);
+    float2 res;
+    res.x = mm;
+    res.y = fast_log2(ll);
+    a.lse[(int64_t)bh * a.rows_pad + i] = res;
 }
 
 // ------------------------------------------------------------------------------------
@@ -327,7 +331,7 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
     constexpr int CPR = D / 8;
     constexpr int CPT = QT * CPR / 256;
     __shared__ __attribute__((aligned(16))) _Float16 lds[2][QT * PITCH];
-    __shared__ float lse_s[2][QT];
+    __shared__ float2 lse_s[2][QT];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
     int bx, by, bz;  // key blocks of one (group, batch entry) stream the same query tiles: same XCD
@@ -355,7 +359,7 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
 
     half8 kf[NA][NT];
     half8 stg[CPT];
-    float stg_lse = 0.f;
+    float2 stg_lse = {0.f, 0.f};
     auto gload = [&](int hs_, int ti_) {  // head and query tile of the stage, counted from the group's first
         const int h = h_begin + hs_, t = t_begin + ti_;
         const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
@@ -366,7 +370,9 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
         }
         if (tid < QT) {
             const int qi = t * QT + tid;
-            stg_lse = (qi < a.q_rows) ? a.lse[((int64_t)b * a.H + h) * a.rows_pad + qi] : INFINITY;
+            stg_lse.x = 0.f;
+            stg_lse.y = INFINITY;  // a row that is not averaged: its probabilities come out as 2^-inf = 0
+            if (qi < a.q_rows) stg_lse = a.lse[((int64_t)b * a.H + h) * a.rows_pad + qi];
         }
     };
     auto lstore = [&](int buf) {
@@ -384,7 +390,7 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
     for (int s = 0; s < nst; ++s) {
         const int t = t_begin + ti;
         if (ti == 0) {  // new head: fetch this wave's key fragments
-            const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)(h_begin + hs) * a.ks_h;
+            const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)kv_head(h_begin + hs, a.kv_group, a.kv_magic) * a.ks_h;
 #pragma unroll
             for (int na = 0; na < NA; ++na) {
                 const _Float16 *row = kp + (int64_t)min(kw0 + na * 32 + r, a.Sk - 1) * a.ks_s + g * 8;
@@ -405,7 +411,11 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
 #pragma unroll
             for (int tt = 0; tt < NT; ++tt)
                 bf[tt] = *reinterpret_cast<const half8 *>(&tile[(nb * 32 + r) * PITCH + tt * 16 + g * 8]);
-            const float nlse = -lse_s[s & 1][nb * 32 + r];
+            // p = 2^((s - m) * c - log2 l).  m is 0 unless pass 1 had to stabilise this row; then the
+            // subtraction comes first, so that scores of any magnitude keep their low bits.
+            const float2 st = lse_s[s & 1][nb * 32 + r];
+            const float nlse = -st.y;
+            const bool shifted = __builtin_amdgcn_ballot_w64(st.x != 0.f) != 0;  // wave-uniform
             const int qmin = t * QT + nb * 32;
             const bool edge = a.causal && (kmax_w > a.k_past + qmin);  // wave-uniform: straddles the diagonal
             const int lim = a.k_past + qmin + r;                       // last key this lane's query sees
@@ -421,6 +431,10 @@ __global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
                     cn[na] = mfma16<BF>(kf[na][tt], bf[tt], cn[na]);
 #pragma unroll
             for (int na = 0; na < NA; ++na) {
+                if (shifted) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) cn[na][i] -= st.x;
+                }
                 if (!edge) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) colacc[na][i] += fast_exp2(fmaf(cn[na][i], a.c, nlse));

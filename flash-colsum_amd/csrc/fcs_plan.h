@@ -43,7 +43,7 @@ struct Plan {
     int f_hg, f_hpg; // head groups, heads per group
     int n_partials;  // slabs summed by the finalize kernel
     // workspace layout (byte offsets, each 256-byte aligned)
-    size_t off_lse;      // float  [B*H][rows_pad]            log2-domain log-sum-exp
+    size_t off_lse;      // float2 [B*H][rows_pad]            row maximum and log2 of the row sum
     size_t off_ml;       // float2 [B*H][n_chunks][rows_pad]  only when n_chunks > 1
     size_t off_partial;  // float  [gh*gq][B][Sk]             only when gh*gq > 1
     size_t total;
@@ -60,7 +60,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     p.bf16 = 0;
     p.causal = causal ? 1 : 0;
     p.k_past = causal ? k_past : 0;
-    p.q_rows = (!causal && cls_n > 0 && cls_n < Sq) ? cls_n : Sq;
+    p.q_rows = (cls_n > 0 && cls_n < Sq) ? cls_n : Sq;
 
     // ---- pass 1
     p.qw = (p.q_rows > 128) ? 64 : 32;
@@ -171,7 +171,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     // ---- workspace
     size_t off = 0;
     p.off_lse = off;
-    off = align256(off + sizeof(float) * (size_t)B * H * p.rows_pad);
+    off = align256(off + 2 * sizeof(float) * (size_t)B * H * p.rows_pad);
     p.off_ml = off;
     if (p.n_chunks > 1) off = align256(off + 2 * sizeof(float) * (size_t)B * H * p.n_chunks * p.rows_pad);
     p.off_partial = off;

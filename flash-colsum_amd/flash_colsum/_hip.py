@@ -9,8 +9,10 @@ The three private launchers keep the names and argument meaning of the reference
 kernel_causal.py:94) and, like them, return fp16; the `*_f32` functions return the
 kernels' fp32 means.
 """
+import collections
 import ctypes
 import os
+import threading
 from typing import Optional
 
 import torch
@@ -59,6 +61,11 @@ def lib() -> ctypes.CDLL:
                 ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                 ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
                 ctypes.c_float, ctypes.c_void_p]
+        cdll.fcs_colsum_general.restype = ctypes.c_int
+        cdll.fcs_colsum_general.argtypes = [
+            ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+            ctypes.c_void_p, ctypes.c_size_t] + [ctypes.c_int] * 8 + [
+            ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64), ctypes.c_float, ctypes.c_void_p]
         got = cdll.fcs_abi_version()
         if got != _ABI_VERSION:
             raise RuntimeError(f"libflashcolsum.so has ABI {got}, this host layer needs {_ABI_VERSION}")
@@ -104,25 +111,42 @@ def workspace_bytes(causal: bool, b: int, h: int, s_q: int, s_k: int, d: int, cl
 
 # One workspace per (device, stream), grown on demand and reused by later calls: calls on one
 # stream execute in order, so the next call may overwrite what the previous one left behind.
-_workspaces = {}
+# The cache holds at most _WS_MAX_ENTRIES streams (least recently used goes first) and nothing
+# above _WS_MAX_CACHED_BYTES: larger workspaces are allocated per call and returned to torch's
+# allocator afterwards.  While a stream is capturing a HIP graph the cache is neither read nor
+# filled: the workspace then comes from the graph's own pool and lives as long as the graph.
+_workspaces = collections.OrderedDict()
+_workspaces_lock = threading.Lock()
 _WS_MIN_BYTES = 1 << 20
+_WS_MAX_CACHED_BYTES = 64 << 20
+_WS_MAX_ENTRIES = 16
 
 
 def _workspace(device: torch.device, stream: int, n_bytes: int) -> torch.Tensor:
+    if n_bytes > _WS_MAX_CACHED_BYTES or torch.cuda.is_current_stream_capturing():
+        return torch.empty((max(n_bytes, 256),), dtype=torch.uint8, device=device)
     key = (device.index, stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < n_bytes:
-        ws = torch.empty((max(n_bytes, _WS_MIN_BYTES),), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
+    with _workspaces_lock:
+        ws = _workspaces.get(key)
+        if ws is None or ws.numel() < n_bytes:
+            ws = torch.empty((max(n_bytes, _WS_MIN_BYTES),), dtype=torch.uint8, device=device)
+            _workspaces[key] = ws
+        _workspaces.move_to_end(key)
+        while len(_workspaces) > _WS_MAX_ENTRIES:
+            _workspaces.popitem(last=False)
     return ws
 
 
 def release_workspaces() -> None:
-    """Drop the cached per-stream workspaces (they are otherwise kept until the process ends)."""
-    _workspaces.clear()
+    """Drop the cached per-stream workspaces (they are otherwise kept until the process ends).
+
+    Kernels already enqueued keep running on the memory they were given; torch's allocator
+    reuses it for later allocations on the same stream in stream order."""
+    with _workspaces_lock:
+        _workspaces.clear()
 
 
-def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16):
+def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16, general=False):
     b, h, s_q, d = q.shape
     s_k = k.shape[2]
     dev = q.device
@@ -134,6 +158,12 @@ def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16):
     ws = _workspace(dev, stream, n_ws)
     qs, ks = _I64x4(*q.stride()), _I64x4(*k.stride())
     bf16 = q.dtype == torch.bfloat16
+    if general:
+        rc = lib().fcs_colsum_general(int(bf16), int(causal), q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr,
+                                      ws.data_ptr(), n_ws, b, h, k.shape[1], s_q, s_k, d, int(cls_n), int(k_past),
+                                      qs, ks, float(scale), stream)
+        _check(rc, "fcs_colsum_general")
+        return (out, out_h) if want_f16 else out
     if causal:
         fn = lib().fcs_colsum_causal_bf16 if bf16 else lib().fcs_colsum_causal_f16
         rc = fn(q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
@@ -146,7 +176,8 @@ def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16):
     return (out, out_h) if want_f16 else out
 
 
-def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n: int, k_past: int, want_f16: bool = False):
+def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n: int, k_past: int, want_f16: bool = False,
+            general: bool = False):
     """Enqueue one call; returns the fp32 means, or (fp32, fp16) when `want_f16`."""
     if q.device.type != "cuda" or k.device != q.device:
         raise ValueError(f"query and key must live on the same GPU, got {q.device} and {k.device}")
@@ -162,9 +193,19 @@ def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n:
     q = _as_kernel_input(q, dtype)
     k = _as_kernel_input(k, dtype)
     if q.device.index == torch.cuda.current_device():
-        return _enqueue(causal, q, k, scale, cls_n, k_past, want_f16)
+        return _enqueue(causal, q, k, scale, cls_n, k_past, want_f16, general)
     with torch.cuda.device(q.device):
-        return _enqueue(causal, q, k, scale, cls_n, k_past, want_f16)
+        return _enqueue(causal, q, k, scale, cls_n, k_past, want_f16, general)
+
+
+def colsum_general(Q: torch.Tensor, K: torch.Tensor, scale: float, causal: bool = False, CLS_N: int = -1,
+                   K_past: Optional[int] = None, want_f16: bool = False):
+    """fcs_colsum_general: (B, S_k) fp32 means (or (fp32, fp16)) for grouped key heads, batched causal
+    calls, causal calls restricted to the first CLS_N rows and non-causal calls with S_q != S_k."""
+    if K_past is None:
+        K_past = max(0, K.shape[2] - Q.shape[2]) if causal else 0
+    return _launch(bool(causal), Q, K, scale, -1 if CLS_N is None or CLS_N < 0 else int(CLS_N), int(K_past), want_f16,
+                   general=True)
 
 
 def colsum_noncausal_f32(Q: torch.Tensor, K: torch.Tensor, scale: float, CLS_N: int = -1) -> torch.Tensor:

@@ -78,4 +78,49 @@ def flash_colsum(
     return _hip._flash_colsum_batched(query, key, scale, CLS_N=cls_n)
 
 
-__all__ = ["flash_colsum", "flash_colsum_f32"]
+def flash_colsum_ext(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    scale: Optional[float] = None,
+    is_causal: bool = False,
+    cls_len: Optional[int] = None,
+    k_past: Optional[int] = None,
+    out_dtype: torch.dtype = torch.float16,
+) -> torch.Tensor:
+    """`flash_colsum` for the shapes the reference operator rejects (explicit opt-in: `flash_colsum`
+    itself keeps raising for them, reference: flash_colsum/ops.py:65-66,79-87,93-97).
+
+    * grouped-query / multi-query attention: key has H_k heads, H_q a multiple of H_k, query head h
+      attends to key head h // (H_q // H_k); the mean runs over all H_q query heads;
+    * causal with any batch size (query (B,H_q,Q_len,D), key (B,H_k,K_len,D), every batch entry aligned
+      alike), and an explicit `k_past` (key j visible to query i  <=>  j <= k_past + i; default
+      max(0, K_len - Q_len));
+    * `cls_len` together with `is_causal`: the mean runs over the first min(cls_len, Q_len) query rows;
+    * non-causal with S_q != S_k (cross-attention shape).
+    Returns (B, S_k) in `out_dtype` (torch.float16 like the reference, or torch.float32).
+    """
+    if query.ndim != 4 or key.ndim != 4:
+        raise ValueError(f"Expected 4D tensors, got query.ndim={query.ndim}, key.ndim={key.ndim}")
+    if query.device.type != "cuda":
+        raise ValueError(f"Flash attention only supports CUDA tensors, got {query.device}")
+    if cls_len is not None and cls_len <= 0:
+        raise ValueError(f"cls_len must be positive, got {cls_len}")
+    bq, hq, sq, dq = query.shape
+    bk, hk, sk, dk = key.shape
+    if bq != bk or dq != dk:
+        raise ValueError(f"Query and key must have same batch size and head_dim, got B_q={bq}, B_k={bk}, D_q={dq}, D_k={dk}")
+    if hk < 1 or hq % hk != 0:
+        raise ValueError(f"Query heads must be a multiple of key heads, got H_q={hq}, H_k={hk}")
+    if k_past is not None and (not is_causal or k_past < 0):
+        raise ValueError("k_past needs is_causal=True and a non-negative value")
+    if out_dtype not in (torch.float16, torch.float32):
+        raise ValueError(f"out_dtype must be torch.float16 or torch.float32, got {out_dtype}")
+    if scale is None:
+        scale = dq ** -0.5
+    cls_n = -1 if cls_len is None else int(cls_len)
+    if out_dtype == torch.float32:
+        return _hip.colsum_general(query, key, float(scale), is_causal, cls_n, k_past)
+    return _hip.colsum_general(query, key, float(scale), is_causal, cls_n, k_past, want_f16=True)[1]
+
+
+__all__ = ["flash_colsum", "flash_colsum_f32", "flash_colsum_ext"]

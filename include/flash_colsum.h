@@ -36,6 +36,7 @@ enum {
     FCS_E_WORKSPACE = -5, /* ws_bytes smaller than fcs_workspace_bytes() for these dims,
                              or ws not 256-byte aligned                                  */
     FCS_E_SCALE = -6,     /* scale is NaN or infinite                                    */
+    FCS_E_DTYPE = -8,     /* fcs_colsum_general: dtype is not FCS_DTYPE_F16 / FCS_DTYPE_BF16 */
     FCS_E_STATIC_LIMIT = -7 /* fcs_colsum_noncausal_f16_static: the call needs more workspace
                                than FCS_STATIC_SCRATCH_BYTES                               */
 };
@@ -52,7 +53,8 @@ const char *fcs_strerror(int code);
 
 /* Bytes of device workspace the launch functions need for these dimensions (row
  * statistics and per-group partial column sums).  `causal` selects the entry point;
- * for the causal entry point pass B = 1.  `cls_n` <= 0 means "all rows".  Returns 0 for
+ * for the fcs_colsum_causal_* entry points pass B = 1 and cls_n = -1 (they average all rows);
+ * H is the number of QUERY heads.  `cls_n` <= 0 means "all rows".  Returns 0 for
  * invalid dimensions.  The workspace needs no initialisation and 256-byte alignment.
  * Replaces the implicit `torch.zeros` accumulator of the reference launchers
  * (reference: flash_colsum/kernel_noncausal_batched.py:104, kernel_noncausal.py:98,
@@ -118,6 +120,27 @@ int fcs_colsum_causal_bf16(const void *q, const void *k, float *out, void *out_f
                            int H, int Q_len, int K_len, int D, int k_past,
                            const int64_t q_strides[4], const int64_t k_strides[4],
                            float scale, void *hip_stream);
+
+/* General form: the shapes the reference operator still rejects, on the same kernels.
+ *   dtype      FCS_DTYPE_F16 or FCS_DTYPE_BF16 (operand type of q and k).
+ *   causal     0 / 1.  With causal != 0 any B >= 1 is accepted: every batch entry is masked with
+ *              the same k_past (the reference raises for B != 1, flash_colsum/ops.py:79-82).
+ *   Hq, Hk     query and key heads, Hq a multiple of Hk: query head h attends to key head
+ *              h / (Hq / Hk), the grouping of grouped-query / multi-query attention (the
+ *              reference raises for Hq != Hk, flash_colsum/ops.py:83-87).  q is (B,Hq,Sq,D),
+ *              k is (B,Hk,Sk,D).
+ *   Sq, Sk     may differ for causal == 0 too (cross-attention shape).
+ *   cls_n      as above, and also honoured for causal != 0: the mean runs over the first
+ *              min(cls_n, Sq) query rows (the reference raises, flash_colsum/ops.py:65-66).
+ *   out        (B,Sk) fp32 means over the Hq * rows averaged rows; out_f16 optional as above.
+ *   ws         fcs_workspace_bytes(causal, B, Hq, Sq, Sk, D, cls_n) bytes.
+ * With Hq == Hk, and B == 1, cls_n < 0 when causal, the result is bit-identical to the entry
+ * points above. */
+enum { FCS_DTYPE_F16 = 0, FCS_DTYPE_BF16 = 1 };
+int fcs_colsum_general(int dtype, int causal, const void *q, const void *k, float *out, void *out_f16,
+                       void *ws, size_t ws_bytes, int B, int Hq, int Hk, int Sq, int Sk, int D,
+                       int cls_n, int k_past, const int64_t q_strides[4], const int64_t k_strides[4],
+                       float scale, void *hip_stream);
 
 #ifdef __cplusplus
 }

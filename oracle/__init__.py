@@ -21,6 +21,11 @@ Parity pins (all in tests/test_oracle.py, none of them re-types the formula):
   * invariances (key shift, scale/Q trade, key/head/row permutations) and the one-hot
     limit at very large scale,
   * committed golden vectors under tests/golden/ written by the pure-Python brute force.
+`colsum_ext_exact` / `colsum_ref_ext` (grouped key heads, batched causal calls, causal calls
+restricted to their first rows, explicit k_past, S_q != S_k) go beyond the reference operator's
+domain; they are pinned by their own brute-force vectors (tests/golden/colsum_ext_golden.npz),
+by scaled_dot_product_attention with enable_gqa, by the harmonic closed form with an explicit
+k_past and by reduction to the pinned functions above when the extension is not used.
 The reference ships no golden vectors or known-answer values for this path.
 """
-from .naive_colsum import naive_colsum, colsum_exact, visible  # noqa: F401
+from .naive_colsum import naive_colsum, colsum_exact, colsum_ext_exact, visible  # noqa: F401

@@ -92,3 +92,53 @@ def colsum_exact(
                     s = s.masked_fill(j > (i + k_past), float("-inf"))
                 out[b] += torch.softmax(s, dim=-1).sum(dim=0)
     return out / (h_n * rows)
+
+
+def colsum_ext_exact(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    scale: Optional[float] = None,
+    is_causal: bool = False,
+    cls_len: Optional[int] = None,
+    k_past: Optional[int] = None,
+    acc_dtype: torch.dtype = torch.float64,
+    row_block: int = 1024,
+) -> torch.Tensor:
+    """Column means for the shapes the reference operator rejects (ops.py:65-66,79-87,93-97).
+
+    The reference defines nothing here; the definition extends baselines.py:35-78 the way
+    grouped-query attention is defined everywhere else:
+      * key head of query head h is h // (H_q // H_k)  (the `repeat_interleave` of key heads);
+      * the causal predicate j <= k_past + i (kernel_causal.py:39,57) applies to every batch
+        entry alike, k_past defaulting to max(0, S_k - S_q) (kernel_causal.py:113);
+      * `cls_len` restricts the mean to the first min(cls_len, S_q) query rows, also when causal;
+      * S_q and S_k may differ without a mask.
+    With H_q == H_k (and B == 1, cls_len None when causal) it is `colsum_exact`.
+    """
+    b_n, h_q, s_q, d = query.shape
+    h_k, s_k = key.shape[1], key.shape[2]
+    if key.shape[0] != b_n or key.shape[3] != d or h_q % h_k != 0:
+        raise ValueError("query (B,Hq,Sq,D) and key (B,Hk,Sk,D) need the same B and D and Hq a multiple of Hk")
+    grp = h_q // h_k
+    if scale is None:
+        scale = 1.0 / (d ** 0.5)
+    rows = s_q
+    if cls_len is not None:
+        if cls_len <= 0:
+            raise ValueError(f"cls_len must be positive, got {cls_len}")
+        rows = min(int(cls_len), s_q)
+    if k_past is None:
+        k_past = max(0, s_k - s_q)
+    out = torch.zeros(b_n, s_k, dtype=acc_dtype)
+    j = torch.arange(s_k).view(1, s_k)
+    for b in range(b_n):
+        for h in range(h_q):
+            kt = key[b, h // grp].to(torch.float32).t().contiguous()
+            for r0 in range(0, rows, row_block):
+                r1 = min(rows, r0 + row_block)
+                s = (query[b, h, r0:r1].to(torch.float32) @ kt).to(acc_dtype) * scale
+                if is_causal:
+                    i = torch.arange(r0, r1).view(-1, 1)
+                    s = s.masked_fill(j > (i + k_past), float("-inf"))
+                out[b] += torch.softmax(s, dim=-1).sum(dim=0)
+    return out / (h_q * rows)

@@ -27,3 +27,19 @@ def golden():
         cases[n] = dict(q=blob[n + "/q"], k=blob[n + "/k"], out=blob[n + "/out"], causal=bool(causal),
                         cls_len=None if cls_len < 0 else cls_len, scale=None if scale != scale else scale)
     return cases
+
+
+@pytest.fixture(scope="session")
+def golden_ext():
+    """Brute-force vectors for the shapes beyond the reference operator's domain (make_golden_ext.py)."""
+    import numpy as np
+
+    blob = np.load(os.path.join(ROOT, "tests", "golden", "colsum_ext_golden.npz"), allow_pickle=False)
+    cases = {}
+    for n in sorted({key.split("/")[0] for key in blob.files}):
+        causal, cls_len, k_past = (int(v) for v in blob[n + "/meta"])
+        scale = float(blob[n + "/scale"][0])
+        cases[n] = dict(q=blob[n + "/q"], k=blob[n + "/k"], out=blob[n + "/out"], causal=bool(causal),
+                        cls_len=None if cls_len < 0 else cls_len, k_past=None if k_past < 0 else k_past,
+                        scale=None if scale != scale else scale)
+    return cases

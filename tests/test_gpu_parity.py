@@ -15,6 +15,7 @@ import torch
 pytestmark = pytest.mark.gpu
 
 ATOL, RTOL = 1e-4, 1e-3
+FACTOR = 16.0  # large-score cases: allowed multiple of the fp32 eager reference's own distance from float64
 
 
 def _inputs(qs, ks, seed=0, same=False):
@@ -478,6 +479,134 @@ def test_public_api_returns_fp16_like_the_reference():
     # non-fp16 inputs are accepted (converted on the device)
     out32 = flash_colsum_f32(q.float().cuda(), k.float().cuda(), is_causal=True)
     _assert_close(out32, _oracle(q, k, is_causal=True), "fp32 inputs")
+
+
+# ---------------------------------------------------------------------------------------
+# the binding stub of INTEGRATION.md, run as written
+# ---------------------------------------------------------------------------------------
+def test_integration_stub_launchers():
+    from flash_colsum import _hip
+    from test_host_api import integration_stub
+
+    ns = integration_stub()
+    q, k = _inputs((3, 4, 200, 64), (3, 4, 200, 64), seed=41)
+    qc, kc = q.cuda(), k.cuda()
+    assert torch.equal(ns["_flash_colsum_batched"](qc, kc, 0.125), _hip._flash_colsum_batched(qc, kc, 0.125))
+    assert torch.equal(ns["_flash_colsum_batched"](qc, kc, 0.125, 2), _hip._flash_colsum_batched(qc, kc, 0.125, 2))
+    assert torch.equal(ns["_flash_colsum_non_batched"](qc[:1], kc[:1], 0.125), _hip._flash_colsum_non_batched(qc[:1], kc[:1], 0.125))
+    assert torch.equal(ns["_flash_colsum_batched"](qc.bfloat16(), kc.bfloat16(), 0.125),
+                       _hip._flash_colsum_batched(qc.bfloat16(), kc.bfloat16(), 0.125))
+    q, k = _inputs((1, 4, 60, 128), (1, 4, 900, 128), seed=42)
+    got = ns["_flash_colsum_causal"](q.cuda(), k.cuda(), 0.1)
+    assert got.shape == (1, 900) and torch.equal(got, _hip._flash_colsum_causal(q.cuda(), k.cuda(), 0.1))
+    with pytest.raises(RuntimeError, match="head dim"):
+        ns["_flash_colsum_batched"](torch.zeros(1, 1, 8, 7, device="cuda"), torch.zeros(1, 1, 8, 7, device="cuda"), 1.0)
+
+
+# ---------------------------------------------------------------------------------------
+# beyond the reference operator's domain: grouped key heads, batched causal, causal cls_len
+# ---------------------------------------------------------------------------------------
+def _run_ext(q, k, **kw):
+    from flash_colsum import flash_colsum_ext
+
+    out = flash_colsum_ext(q.cuda(), k.cuda(), out_dtype=torch.float32, **kw)
+    torch.cuda.synchronize()
+    return out
+
+
+def _oracle_ext(q, k, **kw):
+    from oracle import colsum_ext_exact
+
+    return colsum_ext_exact(q, k, **kw)
+
+
+def test_ext_golden_vectors(golden_ext):
+    for name, c in golden_ext.items():
+        q, k = torch.from_numpy(c["q"]), torch.from_numpy(c["k"])
+        out = _run_ext(q, k, scale=c["scale"], is_causal=c["causal"], cls_len=c["cls_len"], k_past=c["k_past"])
+        _assert_close(out, torch.from_numpy(c["out"]), name)
+
+
+@pytest.mark.parametrize("qs,ks,kw", [
+    ((1, 32, 128, 128), (1, 8, 16384, 128), {"is_causal": True}),             # GQA decode window, 4 query heads per key head
+    ((4, 32, 128, 128), (4, 32, 4096, 128), {"is_causal": True}),             # batched causal
+    ((2, 16, 100, 128), (2, 2, 3000, 128), {"is_causal": True, "cls_len": 37}),
+    ((3, 8, 64, 64), (3, 1, 1000, 64), {"is_causal": True, "k_past": 500}),   # MQA, explicit k_past
+    ((2, 12, 577, 64), (2, 4, 577, 64), {}),                                  # fused path, grouped
+    ((2, 12, 1024, 64), (2, 3, 1024, 64), {}),                                # fused whole tiles, grouped
+    ((8, 16, 2048, 64), (8, 2, 2048, 64), {}),                                # pre-scaled fused variant, grouped
+    ((2, 8, 577, 64), (2, 2, 577, 64), {"cls_len": 1}),                       # few-rows path, grouped
+    ((2, 6, 2500, 64), (2, 2, 2500, 64), {}),                                 # two-pass, grouped
+    ((2, 4, 300, 128), (2, 1, 300, 128), {"scale": -0.1}),
+    ((2, 4, 100, 64), (2, 4, 700, 64), {}),                                   # non-causal, S_q != S_k (fused)
+    ((2, 4, 700, 64), (2, 2, 100, 64), {"cls_len": 3}),                       # ... few rows
+    ((1, 4, 300, 128), (1, 2, 5000, 128), {}),                                # ... two-pass
+    ((1, 6, 3000, 64), (1, 6, 200, 64), {}),                                  # more rows than keys
+])
+def test_ext_shapes(qs, ks, kw):
+    q, k = _inputs(qs, ks, seed=13)
+    _assert_close(_run_ext(q, k, **kw), _oracle_ext(q, k, **kw), f"ext {qs} {ks} {kw}")
+
+
+def test_ext_equals_the_reference_entry_points_bit_for_bit():
+    from flash_colsum import flash_colsum, flash_colsum_ext, flash_colsum_f32
+
+    q, k = _inputs((3, 4, 700, 64), (3, 4, 700, 64), seed=14)
+    assert torch.equal(flash_colsum_ext(q.cuda(), k.cuda(), out_dtype=torch.float32), flash_colsum_f32(q.cuda(), k.cuda()))
+    assert torch.equal(flash_colsum_ext(q.cuda(), k.cuda(), cls_len=2), flash_colsum(q.cuda(), k.cuda(), cls_len=2))
+    q, k = _inputs((1, 4, 90, 128), (1, 4, 2000, 128), seed=15)
+    assert torch.equal(flash_colsum_ext(q.cuda(), k.cuda(), is_causal=True), flash_colsum(q.cuda(), k.cuda(), is_causal=True))
+    # the reference operator itself keeps raising for these shapes
+    with pytest.raises(ValueError, match="batch size 1"):
+        flash_colsum(torch.zeros(2, 4, 8, 64, device="cuda"), torch.zeros(2, 4, 80, 64, device="cuda"), is_causal=True)
+    with pytest.raises(ValueError, match="same heads"):
+        flash_colsum(torch.zeros(1, 4, 8, 64, device="cuda"), torch.zeros(1, 2, 80, 64, device="cuda"), is_causal=True)
+    with pytest.raises(ValueError, match="multiple of key heads"):
+        flash_colsum_ext(torch.zeros(1, 4, 8, 64, device="cuda"), torch.zeros(1, 3, 80, 64, device="cuda"))
+
+
+# ---------------------------------------------------------------------------------------
+# large score magnitudes: |scale * s| * log2(e) in the thousands
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("qs,ks,kw,bf16", [
+    ((3, 2, 1024, 128), (3, 2, 1024, 128), {"cls_len": 1027, "scale": 20.0}, False),
+    ((9, 3, 1024, 96), (9, 3, 1024, 96), {"cls_len": 5, "scale": 20.0}, False),
+    ((1, 5, 100, 32), (1, 5, 2048, 32), {"is_causal": True, "scale": 20.0}, False),
+    ((8, 3, 1024, 64), (8, 3, 1024, 64), {"cls_len": 1027, "scale": 20.0}, False),
+    ((2, 2, 512, 128), (2, 2, 512, 128), {"scale": 20.0}, False),
+    ((8, 1, 1324, 128), (8, 1, 1324, 128), {"scale": 20.0}, True),
+    ((2, 6, 2416, 64), (2, 6, 2416, 64), {"scale": 20.0}, True),
+    ((2, 4, 333, 64), (2, 4, 333, 64), {"cls_len": 2, "scale": 20.0}, False),
+])
+def test_large_score_magnitudes(qs, ks, kw, bf16):
+    """Inputs x4 and scale 20: scale * score reaches +-20000, where one fp32 ulp of a score moves a
+    probability by 1e-3 relative, so the fp32 eager reference itself is 3e-4 .. 1e-3 away from
+    float64.  The matrix pipe adds the 16 products of a step to the accumulator with up to one ulp of
+    error, D/16 steps per score, so the kernels sit D/16 times further out.  Stated bars:
+      * within FACTOR x the fp32 eager reference's own distance from float64, and
+      * within 1.5 x (D_padded / 16) x |scale| x ulp_fp32(max |score|) relative,
+    and the usual 1e-4 / 1e-3 wherever those are larger."""
+    from oracle import naive_colsum
+
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn(qs, generator=g) * 4.0
+    k = torch.randn(ks, generator=g) * 4.0
+    q, k = (q.bfloat16(), k.bfloat16()) if bf16 else (q.half(), k.half())
+    ref = _oracle(q.float(), k.float(), **kw)
+    eager = naive_colsum(q.float(), k.float(), **kw).double()
+    e_abs = (eager - ref).abs().max().item()
+    e_rel = ((eager - ref).abs() / ref.abs().clamp_min(1e-9)).max().item()
+    out = _run(q, k, **kw).cpu().double()
+    assert torch.isfinite(out).all()
+    err = (out - ref).abs()
+    rel = (err / ref.abs().clamp_min(1e-9)).max().item()
+    print(f"large scores {qs} {kw}: kernel abs {err.max().item():.2e} rel {rel:.2e}; fp32 eager abs {e_abs:.2e} rel {e_rel:.2e}")
+    assert err.max().item() <= max(ATOL, FACTOR * e_abs), (err.max().item(), e_abs)
+    assert rel <= max(RTOL, FACTOR * e_rel), (rel, e_rel)
+    s_max = (q.double() @ k.double().transpose(-1, -2)).abs().max().item()
+    steps = (64 if qs[3] <= 64 else 128) // 16
+    ulp = 2.0 ** (np.floor(np.log2(s_max)) - 23)
+    assert rel <= max(RTOL, 1.5 * steps * abs(kw["scale"]) * ulp), (rel, steps, s_max)
 
 
 # ---------------------------------------------------------------------------------------

@@ -148,3 +148,29 @@ def test_missing_library_is_loud(monkeypatch, tmp_path):
     monkeypatch.setattr(_hip, "_LIB_PATH", str(tmp_path / "libflashcolsum.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         _hip.lib()
+
+
+def integration_stub():
+    """The binding stub INTEGRATION.md shows to a maintainer of the reference, executed as written
+    (only the library's file name is replaced by its path in this tree)."""
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    blocks = re.findall(r"```python\n(.*?)```", text, flags=re.S)
+    code = next(b for b in blocks if "_flash_colsum_batched" in b)
+    assert '"libflashcolsum.so"' in code
+    ns = {}
+    exec(compile(code.replace('"libflashcolsum.so"', repr(_hip._LIB_PATH)), "INTEGRATION.md", "exec"), ns)
+    return ns
+
+
+def test_integration_stub_binds_and_reports_errors():
+    ns = integration_stub()
+    lib = ns["_lib"]
+    for name in ("_flash_colsum_batched", "_flash_colsum_non_batched", "_flash_colsum_causal"):
+        assert callable(ns[name])
+    # the error path of the stub: a negative code becomes the library's text
+    p = ctypes.c_void_p(4096)
+    st = (ctypes.c_int64 * 4)(8 * 16 * 64, 16 * 64, 64, 2)
+    rc = lib.fcs_colsum_noncausal_f16(p, p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None)
+    assert rc == -4 and "stride" in lib.fcs_strerror(rc).decode()
+    rc = lib.fcs_colsum_causal_bf16(p, p, p, None, p, 16, 8, 16, 64, 64, 48, st, st, 0.125, None)
+    assert rc < 0 and lib.fcs_strerror(rc).decode()

@@ -12,8 +12,8 @@ import numpy as np
 import pytest
 import torch
 
-from oracle import colsum_exact, naive_colsum, visible
-from oracle.c_ref import colsum_ref
+from oracle import colsum_exact, colsum_ext_exact, naive_colsum, visible
+from oracle.c_ref import colsum_ref, colsum_ref_ext
 
 IMPLS = {
     "torch_naive": lambda q, k, **kw: naive_colsum(q, k, **kw).double().numpy(),
@@ -158,3 +158,89 @@ def test_single_causal_query_sees_every_key():
     want = torch.softmax(s, -1).mean((1, 2)).numpy()
     for impl in IMPLS.values():
         np.testing.assert_allclose(impl(q, k, is_causal=True), want, rtol=3e-6)
+
+
+def test_fp32_reference_leaves_the_bar_at_huge_scores():
+    """Where |scale * score| reaches the tens of thousands one fp32 ulp of a score is worth 1e-3 of a
+    probability: the fp32 eager path (the parity target) is then itself an order of magnitude
+    further from float64 than at ordinary magnitudes, within |scale| * ulp_fp32(max |score|).
+    This is the edge of the domain in which the 1e-3 relative bar can be asked of an fp32 evaluation."""
+    q, k = (_rand((1, 2, 256, 128), 31) * 4).half().float(), (_rand((1, 2, 256, 128), 32) * 4).half().float()
+    exact = colsum_exact(q, k, scale=20.0).numpy()
+    eager = naive_colsum(q, k, scale=20.0).double().numpy()
+    rel = np.max(np.abs(eager - exact) / np.maximum(np.abs(exact), 1e-12))
+    s_max = float((q.double() @ k.double().transpose(-1, -2)).abs().max())
+    ulp = 2.0 ** (math.floor(math.log2(s_max)) - 23)
+    assert 1e-5 < rel <= 20.0 * ulp * 1.5, (rel, s_max)
+    # at ordinary magnitudes the same comparison is at fp32 rounding level
+    q, k = q / 4, k / 4
+    rel = np.max(np.abs(naive_colsum(q, k).double().numpy() - colsum_exact(q, k).numpy()) / colsum_exact(q, k).numpy())
+    assert rel < 2e-6
+
+
+# ---------------------------------------------------------------------------------------
+# beyond the reference operator's domain: grouped key heads, batched causal, causal cls_len,
+# explicit k_past, S_q != S_k
+# ---------------------------------------------------------------------------------------
+EXT_IMPLS = {
+    "torch_ext": lambda q, k, **kw: colsum_ext_exact(q, k, **kw).numpy(),
+    "plain_c_ext": lambda q, k, **kw: colsum_ref_ext(q.numpy(), k.numpy(), **kw),
+}
+
+
+@pytest.mark.parametrize("impl", sorted(EXT_IMPLS))
+def test_ext_against_golden_bruteforce(impl, golden_ext):
+    for name, c in golden_ext.items():
+        q = torch.from_numpy(c["q"].astype(np.float32))
+        k = torch.from_numpy(c["k"].astype(np.float32))
+        got = EXT_IMPLS[impl](q, k, scale=c["scale"], is_causal=c["causal"], cls_len=c["cls_len"], k_past=c["k_past"])
+        np.testing.assert_allclose(got, c["out"], rtol=1e-6, atol=1e-9, err_msg=name)
+
+
+@pytest.mark.parametrize("impl", sorted(EXT_IMPLS))
+def test_ext_reduces_to_the_pinned_oracle(impl, golden):
+    """Without grouping, batching of causal calls or a causal cls_len it is the reference's definition."""
+    for name, c in golden.items():
+        q = torch.from_numpy(c["q"].astype(np.float32))
+        k = torch.from_numpy(c["k"].astype(np.float32))
+        got = EXT_IMPLS[impl](q, k, scale=c["scale"], is_causal=c["causal"], cls_len=c["cls_len"])
+        np.testing.assert_allclose(got, c["out"], rtol=1e-6, atol=1e-9, err_msg=name)
+
+
+@pytest.mark.parametrize("impl", sorted(EXT_IMPLS))
+def test_ext_matches_library_grouped_attention(impl):
+    """scaled_dot_product_attention(enable_gqa=True) with V = I: the library's own grouping of
+    query heads over key heads, with and without its lower-right causal bias, batch of 2."""
+    import torch.nn.functional as F
+    from torch.nn.attention.bias import causal_lower_right
+
+    q, k = _rand((2, 6, 9, 16), 21).double(), _rand((2, 2, 14, 16), 22).double()
+    eye = torch.eye(14, dtype=torch.float64).expand(2, 2, 14, 14)
+    attn = F.scaled_dot_product_attention(q, k, eye, scale=0.3, enable_gqa=True)
+    np.testing.assert_allclose(EXT_IMPLS[impl](q.float(), k.float(), scale=0.3), attn.mean((1, 2)).numpy(), rtol=3e-6)
+    attn = F.scaled_dot_product_attention(q, k, eye, attn_mask=causal_lower_right(9, 14), scale=0.3, enable_gqa=True)
+    np.testing.assert_allclose(EXT_IMPLS[impl](q.float(), k.float(), scale=0.3, is_causal=True),
+                               attn.mean((1, 2)).numpy(), rtol=3e-6, atol=1e-12)
+    # causal cls_len = c: the same matrix restricted to its first c rows
+    np.testing.assert_allclose(EXT_IMPLS[impl](q.float(), k.float(), scale=0.3, is_causal=True, cls_len=4),
+                               attn[:, :, :4].mean((1, 2)).numpy(), rtol=3e-6, atol=1e-12)
+    # the grouping is repeat_interleave of the key heads
+    want = np.stack([colsum_exact(q[b:b + 1].float(), k[b:b + 1].float().repeat_interleave(3, dim=1), scale=0.3,
+                                  is_causal=True).numpy()[0] for b in range(2)])
+    np.testing.assert_allclose(EXT_IMPLS[impl](q.float(), k.float(), scale=0.3, is_causal=True), want, rtol=1e-6)
+
+
+@pytest.mark.parametrize("impl", sorted(EXT_IMPLS))
+@pytest.mark.parametrize("sq,sk,k_past,cls_len", [(5, 12, 3, None), (6, 20, 0, 4), (4, 9, 30, None), (8, 8, 2, 3)])
+def test_ext_causal_closed_form_with_explicit_k_past(impl, sq, sk, k_past, cls_len):
+    """Q = 0: row i is uniform over its min(S_k, k_past + i + 1) visible keys; harmonic sums fix
+    k_past, the <= and the normaliser over the averaged rows."""
+    q, k = torch.zeros(2, 4, sq, 8), _rand((2, 2, sk, 8), 23)
+    out = EXT_IMPLS[impl](q, k, is_causal=True, k_past=k_past, cls_len=cls_len)
+    rows = sq if cls_len is None else min(cls_len, sq)
+    want = np.zeros(sk)
+    for i in range(rows):
+        n = min(sk, k_past + i + 1)
+        want[:n] += 1.0 / n
+    want /= rows
+    np.testing.assert_allclose(out, np.stack([want, want]), rtol=2e-6, atol=1e-12)
