@@ -26,7 +26,8 @@ struct Args {
     float2 *ml;   // [B*H][n_chunks][rows_pad]  (m, l) of each key split
     // pass 2
     int gh, gq, heads_per_group, qtiles_per_group;
-    float *partial;  // [gh*gq][B][Sk]
+    int c_chunk, c_groups, c_upg, c_nrb;  // column pass: keys per block, unit groups, units per group, row blocks per head
+    float *partial;  // [groups][B][Sk]
     float *out;      // [B][Sk]
     _Float16 *out_h; // [B][Sk] or nullptr: the same means rounded to fp16
     float inv_norm;  // 1 / (H * q_rows)
@@ -45,6 +46,9 @@ int launch_colsum(const Plan &p, const Args &a, void *stream);
 hipError_t launch_fused(const Plan &p, const Args &a, hipStream_t st);
 // few-rows path (fcs_fewrows.hip): p.fewrows == 1
 hipError_t launch_fewrows(const Plan &p, const Args &a, hipStream_t st);
+
+// column pass of the two-pass path (fcs_stream.hip)
+hipError_t launch_colstream(const Plan &p, const Args &a, hipStream_t st);
 
 // shared final reduction out = inv_norm * sum of the n_partials slabs (fcs_kernels.hip)
 hipError_t launch_finalize(const Args &a, hipStream_t st);

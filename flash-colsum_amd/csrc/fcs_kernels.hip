@@ -529,22 +529,11 @@ static hipError_t launch_d(const Plan &p, const Args &a, hipStream_t st)
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    if (p.n_chunks > 1) {
-        const dim3 grid((p.rows_pad + 63) / 64, p.B * p.H);
-        hipLaunchKernelGGL(fcs_merge_stats_kernel, grid, dim3(64), 0, st, a);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
     {
-        const dim3 grid(p.n_kblk, p.gh * p.gq, p.B);
-        if (p.kw == 64)
-            hipLaunchKernelGGL((fcs_colsum_kernel<D, 64, BF>), grid, blk, 0, st, a);
-        else
-            hipLaunchKernelGGL((fcs_colsum_kernel<D, 32, BF>), grid, blk, 0, st, a);
-        hipError_t e = hipGetLastError();
+        hipError_t e = launch_colstream(p, a, st);  // merges the key splits of pass 1 itself
         if (e != hipSuccess) return e;
     }
-    if (p.gh * p.gq > 1) {
+    if (p.c_groups > 1) {
         hipError_t e = launch_finalize(a, st);
         if (e != hipSuccess) return e;
     }

@@ -16,6 +16,11 @@ constexpr int kFewRowsMaxRows = 4;      // few-rows path: at most this many aver
 constexpr int kFewRowsMaxScores = 12288; // ... and rows * Sk scores (48 KB of LDS)
 constexpr int kTargetBlocks = 1024; // 256 CUs x 4: enough workgroups to fill the chip twice over
 
+// column pass (fcs_stream.hip): ring slots of 64-key stages and keys per workgroup chunk, sized so
+// that the LDS ring plus one accumulator slice per wave fit (twice per compute unit for 4-wave blocks)
+constexpr int col_ring_slots(int D, int waves) { return (D >= 128 && waves == 4) ? 3 : 4; }
+constexpr int col_chunk_max(int D, int waves) { return (D >= 128 && waves == 4) ? 1536 : 2048; }
+
 struct Plan {
     int B, H, Sq, Sk, D;
     int bf16;    // operands are bf16 instead of fp16 (set by the caller after make_plan)
@@ -33,6 +38,12 @@ struct Plan {
     int n_kblk;
     int gh, gq;      // groups along heads / along staged query tiles
     int heads_per_group, qtiles_per_group;
+    // column pass: grid = (c_nchunks, c_groups, B); a block owns c_chunk keys and walks over c_upg
+    // (head, row block) units
+    int c_nb, c_waves; // 32-row fragments per wave, waves per block: a unit has 32 * c_nb * c_waves rows
+    int c_nrb;         // row blocks per head
+    int c_chunk, c_nchunks;
+    int c_groups, c_upg;
     // fused single-kernel path: non-causal, all keys of a row block fit in one
     // workgroup's registers.  grid = (f_nqblk * B, f_hg)
     int fewrows;     // 1: few-rows path (non-causal, q_rows <= 4): grid = B * f_hg, slabs = f_hg
@@ -116,6 +127,36 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         }
     }
 
+    // ---- column pass (streaming kernel)
+    {
+        if (p.q_rows > 256) { p.c_nb = 2; p.c_waves = 8; }
+        else if (p.q_rows > 128) { p.c_nb = 2; p.c_waves = 4; }
+        else { p.c_nb = 1; p.c_waves = 4; }
+        const int block_rows = 32 * p.c_nb * p.c_waves;
+        p.c_nrb = ceil_div(p.q_rows, block_rows);
+        const long units = (long)H * p.c_nrb;
+        const int chunk_max = col_chunk_max(D, p.c_waves);
+        const long target = (p.c_waves == 8) ? kComputeUnits : 2 * kComputeUnits;
+        int chunk = ceil_div(Sk, kStageKeys) * kStageKeys;
+        if (chunk > chunk_max) chunk = chunk_max;
+        int nchunks = ceil_div(Sk, chunk);
+        long groups = (target + (long)B * nchunks - 1) / ((long)B * nchunks);
+        if (groups > units) {
+            // one unit per block is still too few blocks: shorter chunks (at least four stages each)
+            groups = units;
+            const long want = (target + (long)B * units - 1) / ((long)B * units);
+            int c = ceil_div(ceil_div(Sk, (int)(want < 1 ? 1 : want)), kStageKeys) * kStageKeys;
+            if (c < 4 * kStageKeys) c = 4 * kStageKeys;
+            if (c < chunk) chunk = c;
+            nchunks = ceil_div(Sk, chunk);
+        }
+        if (groups < 1) groups = 1;
+        p.c_chunk = chunk;
+        p.c_nchunks = nchunks;
+        p.c_upg = (int)((units + groups - 1) / groups);
+        p.c_groups = (int)((units + p.c_upg - 1) / p.c_upg);
+    }
+
     // ---- few-rows path: a batch of matrix-vector products, one workgroup per (batch entry, head group)
     p.fewrows = 0;
     p.fused = 0;
@@ -133,7 +174,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     }
 
     // ---- fused path
-    p.n_partials = p.gh * p.gq;
+    p.n_partials = p.c_groups;
     if (!causal && Sk <= kFusedMaxKeys && D == 64) {
         p.fused = 1;
         const int tiles = ceil_div(Sk, 32);
@@ -175,7 +216,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     p.off_ml = off;
     if (p.n_chunks > 1) off = align256(off + 2 * sizeof(float) * (size_t)B * H * p.n_chunks * p.rows_pad);
     p.off_partial = off;
-    if (p.gh * p.gq > 1) off = align256(off + sizeof(float) * (size_t)p.gh * p.gq * B * Sk);
+    if (p.c_groups > 1) off = align256(off + sizeof(float) * (size_t)p.c_groups * B * Sk);
     p.total = off;
     return true;
 }

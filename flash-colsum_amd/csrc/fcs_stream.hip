@@ -1,0 +1,413 @@
+// Attention column means on gfx950 (MI355X): the column pass of the general two-pass path.
+//
+// Given the row statistics of pass 1 (row maximum m_i and l_i = sum_j 2^((s_ij - m_i) * c),
+// c = scale * log2(e)), this kernel adds up  p_ij = 2^((s_ij - m_i) * c - log2 l_i)  over heads and
+// query rows for every key j.
+//
+// Orientation  S = Q_tile * K_tile^T  on v_mfma_f32_32x32x16: a lane owns ONE key (column
+// lane % 32 of the tile) and 16 query rows of it in its accumulator registers.
+//   * Q is the stationary operand: a wave keeps 32 * NB query rows of one head in registers.
+//   * The per-row constant  n_i = -log2(l_i) / c  enters the matrix pipe as the INITIAL
+//     accumulator value of the row, so the scores leave the MFMAs as  s_ij + n_i  and
+//     p_ij = 2^(c * (s_ij + n_i))  costs one multiply and one v_exp_f32.  (Rows that pass 1 had
+//     to stabilise, m_i != 0, are rare: a unit that holds one starts its accumulators at 0, so
+//     that its scores carry the very bits pass 1 saw, subtracts m_i before the scale and
+//     log2 l_i after it.)
+//   * Summing p over the rows of a tile is in-lane; the two half-waves (which hold different
+//     rows of the same keys) are added with v_permlane32_swap, and the wave adds its total for
+//     the stage's keys into ITS OWN slice of an LDS accumulator with ds_add_f32.  One lane is the
+//     only writer of an address, stage after stage, so the order of additions is fixed.
+//   * K is streamed: the waves of a workgroup share 64-key stages that they fetch with
+//     global_load_lds_dwordx4 straight into an LDS ring, several stages ahead, XOR-swizzled so
+//     that the operand reads (ds_read_b128, 32 rows a row pitch apart) are conflict-free.  One
+//     workgroup barrier per stage; the DMA is waited for by hand with s_waitcnt vmcnt(n).
+// A workgroup owns a chunk of keys (at most kColChunkMax, the LDS accumulator) and walks over a
+// group of (head, row block) units, re-streaming its chunk for each; at the end the waves'
+// slices are added in wave order and written as one partial slab (or the means directly, when
+// there is a single group).  Causal alignment  j <= k_past + i  (reference:
+// flash_colsum/kernel_causal.py:39,57,113): the stage loop stops at the last key any row of the
+// unit sees, only stages on the diagonal (or past the last key) take the masked code path.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fcs_device.h"
+#include "fcs_kernels.h"
+
+namespace fcs {
+
+namespace {
+
+#define FCS_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
+#define FCS_WAIT_LGKM0() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
+
+// 64 lanes x 16 bytes from global memory straight into LDS: lane L's piece lands at dst + 16 * L
+// (dst is wave-uniform)
+__device__ __forceinline__ void dma16(const char *src, char *dst)
+{
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                     (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+}
+
+// workgroup barrier that also orders this wave's LDS accesses around it (the bare s_barrier
+// intrinsic is neither a fence for the compiler nor a wait for outstanding LDS writes)
+__device__ __forceinline__ void block_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+__device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+__device__ __forceinline__ uint32_t lds_addr(const void *p)
+{
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
+}
+
+// position swizzle of the 16-byte pieces of a stage row: rows a row pitch apart must not share banks
+template <int D>
+__device__ __forceinline__ int row_swizzle(int row)
+{
+    return D == 64 ? ((row >> 1) & 7) : (row & 15);
+}
+
+}  // namespace
+
+template <int D, int NB, int WAVES, bool BF>
+__global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args a)
+{
+    constexpr int THREADS = 64 * WAVES;
+    constexpr int NT = D / 16;                 // MFMA steps along the head dim
+    constexpr int KT = kStageKeys;             // 64 keys per stage
+    constexpr int NA = KT / 32;                // key fragments per stage
+    constexpr int ROWS_W = 32 * NB;            // query rows per wave
+    constexpr int BLOCK_ROWS = WAVES * ROWS_W;
+    constexpr int ROW_BYTES = D * 2;
+    constexpr int PPR = D / 8;                 // 16-byte pieces per row
+    constexpr int STAGE_BYTES = KT * ROW_BYTES;
+    constexpr int IPW = KT * PPR / THREADS;    // DMA instructions per wave per stage
+    constexpr int NS = col_ring_slots(D, WAVES);
+    constexpr int CHUNK = col_chunk_max(D, WAVES);
+    static_assert(IPW >= 1 && KT * PPR == IPW * THREADS, "a stage is a whole number of DMA instructions per wave");
+    static_assert(NS >= 3, "the ring holds the stage in use, the next one and at least one in flight");
+    __shared__ __attribute__((aligned(16))) char ring[NS * STAGE_BYTES];
+    __shared__ __attribute__((aligned(16))) float colw[WAVES * CHUNK];  // per-wave column sums of the chunk
+    __shared__ __attribute__((aligned(16))) float nl_s[BLOCK_ROWS];     // per-row constants of the current unit
+    __shared__ __attribute__((aligned(16))) float lg_s[BLOCK_ROWS];     // log2 l_i, used by units with stabilised rows
+    __shared__ __attribute__((aligned(16))) float cm_s[BLOCK_ROWS];     // -m_i of those units
+    __shared__ int shift_s[WAVES];                                       // per wave: one of its rows is stabilised
+
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int cx, grp, b;  // chunks of one (group, batch entry) stream the same Q: neighbours in launch order
+    xcd_contiguous_block(cx, grp, b);
+    const int c0 = cx * a.c_chunk;                     // first key of the chunk
+    const int c1 = min(a.Sk, c0 + a.c_chunk);          // one past its last key
+    const int u_begin = grp * a.c_upg, u_end = min(a.H * a.c_nrb, u_begin + a.c_upg);
+    const float cmul = (a.c == 0.f) ? 1.f : a.c;       // scale 0: Q is zeroed instead and n_i = -log2 l_i
+
+    // ---- this wave's slice of the column accumulator
+    float *colw_w = colw + wave * CHUNK;
+    for (int i = lane * 4; i < CHUNK; i += 256) *reinterpret_cast<floatx4 *>(colw_w + i) = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // ---- DMA geometry: piece P of a stage goes to LDS byte 16 * P; it is piece pos ^ swizzle(row)
+    // of stage row `row`, so that row r keeps piece p at position p ^ swizzle(r)
+    uint32_t g_off[IPW];   // byte offset of this lane's piece from the stage's first key row (dense stage)
+#pragma unroll
+    for (int j = 0; j < IPW; ++j) {
+        const int P = (wave * IPW + j) * 64 + lane;
+        const int row = P / PPR, pos = P % PPR;
+        g_off[j] = (uint32_t)row * (uint32_t)(a.ks_s * 2) + (uint32_t)((pos ^ row_swizzle<D>(row)) * 16);
+    }
+    char *ring_w = ring + wave * (IPW * 1024);  // where this wave's pieces of a stage land inside a slot
+    // operand read-back: lane (n, g) takes, for MFMA step t, piece 2t + g of row n (+ 32 per key fragment)
+    uint32_t take[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+        take[t] = lds_addr(ring) + (uint32_t)(n * ROW_BYTES + (((2 * t + g) ^ row_swizzle<D>(n)) * 16));
+
+    for (int u = u_begin; u < u_end; ++u) {
+        const int h = u / a.c_nrb, rb = u - h * a.c_nrb;
+        const int row0 = rb * BLOCK_ROWS;                        // first query row of the unit
+        const int rows_end = min(a.q_rows, row0 + BLOCK_ROWS);   // one past its last averaged row
+        // keys of the chunk that some row of the unit sees
+        int kend = c1;
+        if (a.causal) kend = min(kend, a.k_past + rows_end);
+        const int nst = (kend > c0) ? (kend - c0 + KT - 1) / KT : 0;
+        if (nst == 0) continue;  // block-uniform
+
+        // ---- per-row constants, merged over the key splits of pass 1
+        {
+            const int qi = row0 + tid;
+            float nl = -INFINITY;  // a row that is not averaged: every p comes out as 2^-inf = 0
+            float mm = 0.f, lg = 0.f;
+            if (tid < BLOCK_ROWS && qi < a.q_rows) {
+                const int64_t bh = (int64_t)b * a.H + h;
+                if (a.n_chunks == 1) {
+                    const float2 v = a.lse[bh * a.rows_pad + qi];
+                    mm = v.x;
+                    lg = v.y;
+                } else {
+                    const float2 *p = a.ml + bh * a.n_chunks * a.rows_pad + qi;
+                    mm = kNegBig * 4.f;
+                    float ll = 0.f;
+                    for (int ch = 0; ch < a.n_chunks; ++ch) {  // fixed order: bit-reproducible
+                        const float2 v = p[(int64_t)ch * a.rows_pad];
+                        const float mn = fmaxf(mm, v.x);
+                        ll = ll * fast_exp2((mm - mn) * a.c) + v.y * fast_exp2((v.x - mn) * a.c);
+                        mm = mn;
+                    }
+                    lg = fast_log2(ll);
+                }
+                nl = (a.c == 0.f) ? -lg : -lg / a.c;
+            }
+            // a stabilised row anywhere in the unit switches the whole unit to the two-constant form
+            const bool sh = __builtin_amdgcn_ballot_w64(mm != 0.f) != 0;
+            if (lane == 0) shift_s[wave] = sh ? 1 : 0;
+            if (tid < BLOCK_ROWS) {
+                nl_s[tid] = nl;
+                lg_s[tid] = lg;
+                cm_s[tid] = (nl == -INFINITY) ? -INFINITY : -mm;
+            }
+        }
+
+        // ---- stationary operand: this wave's query rows of head h
+        const int qw0 = row0 + wave * ROWS_W;
+        half8 qf[NB][NT];
+        {
+            const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const _Float16 *row = qp + (int64_t)min(qw0 + nb * 32 + n, a.Sq - 1) * a.qs_s + g * 8;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    half8 v = load8(row + t * 16);
+                    if (a.negate) v = flip_sign(v);
+                    if (a.c == 0.f) v = half8{0, 0, 0, 0, 0, 0, 0, 0};
+                    qf[nb][t] = v;
+                }
+            }
+        }
+        const char *kp = reinterpret_cast<const char *>(a.k + (int64_t)b * a.ks_b +
+                                                        (int64_t)kv_head(h, a.kv_group, a.kv_magic) * a.ks_h);
+        const int64_t k_row_b = a.ks_s * 2;
+
+        // stage `st` of the unit into ring slot `slot` (stages past the last one repeat it, so that the
+        // number of DMA instructions in flight at every wait is a compile-time constant)
+        auto fetch_stage = [&](int st, int slot) {
+            const int kb = c0 + min(st, nst - 1) * KT;
+            char *dst = ring_w + slot * STAGE_BYTES;
+            if (kb + KT <= a.Sk) {  // whole stage inside the tensor (wave-uniform)
+                const char *src = kp + (int64_t)kb * k_row_b;
+#pragma unroll
+                for (int j = 0; j < IPW; ++j) dma16(src + g_off[j], dst + j * 1024);
+            } else {  // rows past the last key re-read it; the consumer masks them
+                int lane_o = lane;
+                asm volatile("" : "+v"(lane_o));  // formed here, not kept in registers through the stream
+#pragma unroll
+                for (int j = 0; j < IPW; ++j) {
+                    const int P = (wave * IPW + j) * 64 + lane_o;
+                    const int row = P / PPR, pos = P % PPR;
+                    dma16(kp + (int64_t)min(kb + row, a.Sk - 1) * k_row_b + (pos ^ row_swizzle<D>(row)) * 16, dst + j * 1024);
+                }
+            }
+        };
+
+        // key fragment `na` of the stage in `slot` as MFMA B operand.  Inline assembly: the compiler
+        // would make an ordinary LDS read wait for ALL outstanding DMA (vmcnt(0)).
+        auto take_frag = [&](int slot, int na, half8 (&kf)[NT]) {
+            const uint32_t off = (uint32_t)(slot * STAGE_BYTES + na * 32 * ROW_BYTES);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const uint32_t ad = take[t] + off;
+                asm volatile("ds_read_b128 %0, %1" : "=v"(kf[t]) : "v"(ad) : "memory");
+            }
+        };
+        auto frag_wait = [&](half8 (&kf)[NT]) {
+            if constexpr (NT == 4)
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kf[0]), "+v"(kf[1]), "+v"(kf[2]), "+v"(kf[3])::"memory");
+            else {
+#pragma unroll
+                for (int t0 = 0; t0 < NT; t0 += 8)
+                    asm volatile("s_waitcnt lgkmcnt(0)"
+                                 : "+v"(kf[t0]), "+v"(kf[t0 + 1]), "+v"(kf[t0 + 2]), "+v"(kf[t0 + 3]), "+v"(kf[t0 + 4]),
+                                   "+v"(kf[t0 + 5]), "+v"(kf[t0 + 6]), "+v"(kf[t0 + 7])::"memory");
+            }
+        };
+
+        // ---- prologue: NS - 1 stages in flight; stages 0 and 1 must have landed before the first barrier
+#pragma unroll
+        for (int st = 0; st < NS - 1; ++st) fetch_stage(st, st);
+        FCS_WAIT_VM((NS - 3) * IPW);
+        block_sync();  // also publishes nl_s
+
+        bool shifted = false;  // block-uniform: some row of the unit was stabilised by pass 1
+        {
+            int f = 0;
+            const uint32_t ad = lds_addr(shift_s) + (uint32_t)((lane % WAVES) * 4);
+            asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(f) : "v"(ad) : "memory");
+            shifted = __builtin_amdgcn_ballot_w64(f != 0) != 0;
+        }
+        floatx16 cinit[NB];  // row constants in accumulator layout: register i <-> row 8*(i/4) + 4*g + i%4
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                floatx4 v;  // inline assembly for the same reason as the operand reads below
+                const uint32_t ad = lds_addr(nl_s) + (uint32_t)((wave * ROWS_W + nb * 32 + 8 * i4 + 4 * g) * 4);
+                asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(ad) : "memory");
+#pragma unroll
+                for (int j = 0; j < 4; ++j) cinit[nb][4 * i4 + j] = shifted ? 0.f : v[j];
+            }
+
+        // rows of this wave relative to the causal diagonal; non-causal: every key below Sk is visible
+        const int kp_eff = a.causal ? a.k_past : 0x3fffffff - a.Sq;
+        const int thr_wave_min = a.causal ? min(a.k_past + qw0, a.Sk - 1) : a.Sk - 1;   // last key EVERY row of the wave sees
+        const int thr_wave_max = a.causal ? a.k_past + qw0 + ROWS_W - 1 : 0x3fffffff;  // last key ANY row of the wave sees
+
+        half8 kf[NT];
+        take_frag(0, 0, kf);
+        int slot = 0;
+        for (int st = 0; st < nst; ++st) {
+            const int kb = c0 + st * KT;
+            if (st > 0) {
+                // stage st + 1 has landed (this wave's pieces; the barrier extends that to everyone's), and
+                // every wave is done reading stage st - 1, whose slot takes the next fetch
+                FCS_WAIT_VM((NS - 3) * IPW);
+                block_barrier();
+            }
+            {
+                int free_slot = slot - 1;
+                if (free_slot < 0) free_slot += NS;
+                fetch_stage(st + NS - 1, free_slot);
+            }
+            const bool hidden = kb > thr_wave_max;  // wave-uniform: no row of this wave sees any key of the stage
+            float colt[NA];
+#pragma unroll
+            for (int na = 0; na < NA; ++na) {
+                floatx16 acc[NB];
+                frag_wait(kf);
+                if (!hidden) {
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) {
+                        acc[nb] = mfma16<BF>(qf[nb][0], kf[0], cinit[nb]);
+#pragma unroll
+                        for (int t = 1; t < NT; ++t) acc[nb] = mfma16<BF>(qf[nb][t], kf[t], acc[nb]);
+                    }
+                }
+                // the next fragment is read back while the matrix pipe and the exponents run
+                if (na + 1 < NA) {
+                    take_frag(slot, na + 1, kf);
+                } else {
+                    int nslot = slot + 1;
+                    if (nslot == NS) nslot = 0;
+                    take_frag(nslot, 0, kf);
+                }
+                float cp[4] = {0.f, 0.f, 0.f, 0.f};
+                if (!hidden) {
+                    const int key = kb + na * 32 + n;
+                    const bool edge = kb + na * 32 + 31 > thr_wave_min;  // wave-uniform
+                    if (shifted) {
+                        // rare: the accumulators started at 0, so the scores carry the very bits pass 1 saw;
+                        // m_i is subtracted before the scale and log2 l_i after it
+                        int rel = (key < a.Sk) ? key - kp_eff - (qw0 + 4 * g) : 0x3fffffff;
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                            for (int i4 = 0; i4 < 4; ++i4) {
+                                floatx4 l4, m4;
+                                const uint32_t ro = (uint32_t)((wave * ROWS_W + nb * 32 + 8 * i4 + 4 * g) * 4);
+                                const uint32_t ad = lds_addr(lg_s) + ro, am = lds_addr(cm_s) + ro;
+                                asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
+                                             : "=&v"(l4), "=&v"(m4)
+                                             : "v"(ad), "v"(am)
+                                             : "memory");
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) {
+                                    const float p = fast_exp2(fmaf(acc[nb][4 * i4 + j] + m4[j], cmul, -l4[j]));
+                                    cp[j] += (rel <= nb * 32 + 8 * i4 + j) ? p : 0.f;
+                                }
+                            }
+                    } else if (!edge) {
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) cp[i & 3] += fast_exp2(acc[nb][i] * cmul);
+                    } else {
+                        // visible  <=>  key < Sk  and  key - k_past - (row of register i) <= 0
+                        int rel = (key < a.Sk) ? key - kp_eff - (qw0 + 4 * g) : 0x3fffffff;
+                        asm volatile("" : "+v"(rel));
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) {
+                                const float p = fast_exp2(acc[nb][i] * cmul);
+                                cp[i & 3] += (rel <= nb * 32 + 8 * (i >> 2) + (i & 3)) ? p : 0.f;
+                            }
+                    }
+                }
+                colt[na] = (cp[0] + cp[1]) + (cp[2] + cp[3]);
+            }
+            // the two half-waves hold different rows of the same keys: add them, then the lower half adds
+            // the stage's totals into this wave's slice of the chunk accumulator
+            if (!hidden) {
+#pragma unroll
+                for (int na = 0; na < NA; ++na) {
+                    const int vi = __builtin_bit_cast(int, colt[na]);
+                    const auto sw = __builtin_amdgcn_permlane32_swap(vi, vi, false, false);
+                    const float other = __builtin_bit_cast(float, g == 0 ? sw[1] : sw[0]);
+                    colt[na] += other;
+                }
+                if (g == 0) {
+                    const uint32_t ad = lds_addr(colw_w) + (uint32_t)((kb - c0 + n) * 4);
+                    asm volatile("ds_add_f32 %0, %1" ::"v"(ad), "v"(colt[0]) : "memory");
+                    asm volatile("ds_add_f32 %0, %1 offset:128" ::"v"(ad), "v"(colt[1]) : "memory");
+                }
+            }
+            slot = (slot + 1 == NS) ? 0 : slot + 1;
+        }
+        // the look-ahead fetches and the operand read-back issued past the last stage must be over before
+        // the next unit reuses the ring (and nl_s)
+        FCS_WAIT_VM(0);
+        frag_wait(kf);
+        block_sync();
+    }
+
+    // ---- add the waves' slices in wave order and store
+    block_sync();
+    const bool direct = (a.c_groups == 1);
+    for (int i = tid; i < c1 - c0; i += THREADS) {
+        float v = colw[i];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) v += colw[w * CHUNK + i];
+        const int64_t o = (int64_t)b * a.Sk + c0 + i;
+        if (direct) {
+            a.out[o] = v * a.inv_norm;
+            if (a.out_h) a.out_h[o] = (_Float16)(v * a.inv_norm);
+        } else {
+            a.partial[(int64_t)grp * a.B * a.Sk + o] = v;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------
+template <int D, int NB, int WAVES, bool BF>
+static hipError_t launch_cfg(const Plan &p, const Args &a, hipStream_t st)
+{
+    const dim3 grid(p.c_nchunks, p.c_groups, p.B);
+    hipLaunchKernelGGL((fcs_colstream_kernel<D, NB, WAVES, BF>), grid, dim3(64 * WAVES), 0, st, a);
+    return hipGetLastError();
+}
+
+template <int D, bool BF>
+static hipError_t launch_colstream_d(const Plan &p, const Args &a, hipStream_t st)
+{
+    if (p.c_nb == 2 && p.c_waves == 8) return launch_cfg<D, 2, 8, BF>(p, a, st);
+    if (p.c_nb == 2 && p.c_waves == 4) return launch_cfg<D, 2, 4, BF>(p, a, st);
+    if (p.c_nb == 1 && p.c_waves == 4) return launch_cfg<D, 1, 4, BF>(p, a, st);
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_colstream(const Plan &p, const Args &a, hipStream_t st)
+{
+    if (p.bf16) return (p.D == 64) ? launch_colstream_d<64, true>(p, a, st) : launch_colstream_d<128, true>(p, a, st);
+    return (p.D == 64) ? launch_colstream_d<64, false>(p, a, st) : launch_colstream_d<128, false>(p, a, st);
+}
+
+}  // namespace fcs
