@@ -85,8 +85,6 @@ int run(int bf16, int causal, const void *q, const void *k, float *out, void *ou
     char *w = static_cast<char *>(ws);
     a.lse = reinterpret_cast<float2 *>(w + p.off_lse);
     a.ml = reinterpret_cast<float2 *>(w + p.off_ml);
-    a.gh = p.gh; a.gq = p.gq;
-    a.heads_per_group = p.heads_per_group; a.qtiles_per_group = p.qtiles_per_group;
     a.c_chunk = p.c_chunk; a.c_groups = p.c_groups; a.c_upg = p.c_upg; a.c_nrb = p.c_nrb;
     a.partial = reinterpret_cast<float *>(w + p.off_partial);
     a.out = out;

@@ -25,7 +25,6 @@ struct Args {
                   //                            unstabilised path) and log2 of sum_j 2^((s_ij - m) * c)
     float2 *ml;   // [B*H][n_chunks][rows_pad]  (m, l) of each key split
     // pass 2
-    int gh, gq, heads_per_group, qtiles_per_group;
     int c_chunk, c_groups, c_upg, c_nrb;  // column pass: keys per block, unit groups, units per group, row blocks per head
     float *partial;  // [groups][B][Sk]
     float *out;      // [B][Sk]

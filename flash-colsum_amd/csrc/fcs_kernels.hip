@@ -1,18 +1,16 @@
-// Attention column means on gfx950 (MI355X): the general two-pass path.
+// Attention column means on gfx950 (MI355X): the general two-pass path, pass 1 and the final
+// reduction.
 //
-// Both passes compute 32x32 score tiles  S^T = K_tile * Q_tile^T  on
-// v_mfma_f32_32x32x16_f16, so that a lane owns ONE query (column l%32 of the tile) and
-// holds 16 keys of it in its accumulator registers (key row 8*(r/4) + 4*(l/32) + r%4).
-//
-//   pass 1 (fcs_rowstats_kernel)  Q tile stationary in registers, K streamed through LDS.
-//          Row max and sum-of-exp are then plain in-lane running scalars; the two
-//          half-waves are combined once at the end.  Emits lse2[i] = log2 sum_j 2^(c*s_ij)
-//          (c = scale*log2(e)), or a partial (max,sum) per key split.
-//   pass 2 (fcs_colsum_kernel)    K tile stationary in registers, Q (+ lse2) streamed
-//          through LDS.  p_ij = 2^(c*s_ij - lse2[i]) is one FMA and one v_exp_f32; each
-//          lane adds it into a per-key register, and the 32 query lanes are summed once
-//          at the very end.  No atomics: every partial has exactly one writer and the
-//          groups are added in a fixed order by fcs_finalize_kernel.
+//   pass 1 (fcs_rowstats_kernel, here)  32x32 score tiles  S^T = K_tile * Q_tile^T  on
+//          v_mfma_f32_32x32x16_f16: a lane owns ONE query (column l%32 of the tile) and holds 16
+//          keys of it in its accumulator registers (key row 8*(r/4) + 4*(l/32) + r%4).  Q tile
+//          stationary in registers, K streamed through LDS.  Row max and sum-of-exp are then plain
+//          in-lane running scalars; the two half-waves are combined once at the end.  Emits per row
+//          (m, log2 l) with l = sum_j 2^((s_ij - m) * c), c = scale*log2(e), or (m, l) per key split.
+//   pass 2 (fcs_colstream_kernel, fcs_stream.hip)  column sums of 2^((s_ij - m_i) * c - log2 l_i),
+//          one partial slab per group of (head, row block) units.
+//   fcs_finalize_kernel (here) adds the slabs in a fixed order: no atomics anywhere, every
+//          partial has exactly one writer.
 //
 // The fragment <-> head-dim mapping (which 8 channels a lane feeds to which MFMA step) is
 // the same for both operands, which is all the contraction needs.
@@ -282,199 +280,6 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
             } else {
                 v.y = ll;
                 a.ml[((int64_t)bh * a.n_chunks + chunk) * a.rows_pad + qi] = v;
-            }
-        }
-    }
-}
-
-// merge the per-split (max, sum) partials of pass 1 into (max, log2 sum): one thread per row, eight partials
-// loaded at a time and folded in split order (fixed order: bit-reproducible)
-__global__ __launch_bounds__(64) void fcs_merge_stats_kernel(const Args a)
-{
-    const int i = blockIdx.x * 64 + threadIdx.x;
-    const int bh = blockIdx.y;
-    if (i >= a.rows_pad) return;
-    const float2 *p = a.ml + (int64_t)bh * a.n_chunks * a.rows_pad + i;
-    float mm = kNegBig * 4.f, ll = 0.f;
-    for (int c0 = 0; c0 < a.n_chunks; c0 += 8) {
-        float2 v[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            v[j].x = kNegBig * 4.f;
-            v[j].y = 0.f;
-            if (c0 + j < a.n_chunks) v[j] = p[(int64_t)(c0 + j) * a.rows_pad];
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float mn = fmaxf(mm, v[j].x);
-            ll = ll * fast_exp2((mm - mn) * a.c) + v[j].y * fast_exp2((v[j].x - mn) * a.c);
-            mm = mn;
-        }
-    }
-    float2 res;
-    res.x = mm;
-    res.y = fast_log2(ll);
-    a.lse[(int64_t)bh * a.rows_pad + i] = res;
-}
-
-// ------------------------------------------------------------------------------------
-// pass 2: column sums of p_ij = 2^(c*s_ij - lse2[i])
-// ------------------------------------------------------------------------------------
-template <int D, int KW, bool BF>
-__global__ __launch_bounds__(256, 2) void fcs_colsum_kernel(const Args a)
-{
-    constexpr int NA = KW / 32;
-    constexpr int NT = D / 16;
-    constexpr int QT = kStageRows;
-    constexpr int NB = QT / 32;
-    constexpr int PITCH = D + 8;
-    constexpr int CPR = D / 8;
-    constexpr int CPT = QT * CPR / 256;
-    __shared__ __attribute__((aligned(16))) _Float16 lds[2][QT * PITCH];
-    __shared__ float2 lse_s[2][QT];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
-    int bx, by, bz;  // key blocks of one (group, batch entry) stream the same query tiles: same XCD
-    xcd_contiguous_block(bx, by, bz);
-    const int b = bz;
-    const int grp = by, gh_i = grp / a.gq, gq_i = grp - gh_i * a.gq;
-    const int k0 = bx * (4 * KW);
-    const int kw0 = k0 + wave * KW;
-    const int kmax_w = kw0 + KW - 1;
-
-    const int h_begin = gh_i * a.heads_per_group;
-    const int h_end = min(a.H, h_begin + a.heads_per_group);
-    const int n_qt = (a.q_rows + QT - 1) / QT;
-    int t_begin = gq_i * a.qtiles_per_group;
-    const int t_end = min(n_qt, t_begin + a.qtiles_per_group);
-    if (a.causal) t_begin = max(t_begin, max(0, k0 - a.k_past) / QT);  // earlier rows see none of these keys
-    const int nt = max(0, t_end - t_begin);
-    const int nst = nt * max(0, h_end - h_begin);
-
-    floatx16 colacc[NA];
-#pragma unroll
-    for (int na = 0; na < NA; ++na)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) colacc[na][i] = 0.f;
-
-    half8 kf[NA][NT];
-    half8 stg[CPT];
-    float2 stg_lse = {0.f, 0.f};
-    auto gload = [&](int hs_, int ti_) {  // head and query tile of the stage, counted from the group's first
-        const int h = h_begin + hs_, t = t_begin + ti_;
-        const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
-#pragma unroll
-        for (int i = 0; i < CPT; ++i) {
-            const int c = tid + i * 256, row = c / CPR, col = (c % CPR) * 8;
-            stg[i] = load8(qp + (int64_t)min(t * QT + row, a.Sq - 1) * a.qs_s + col);
-        }
-        if (tid < QT) {
-            const int qi = t * QT + tid;
-            stg_lse.x = 0.f;
-            stg_lse.y = INFINITY;  // a row that is not averaged: its probabilities come out as 2^-inf = 0
-            if (qi < a.q_rows) stg_lse = a.lse[((int64_t)b * a.H + h) * a.rows_pad + qi];
-        }
-    };
-    auto lstore = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < CPT; ++i) {
-            const int c = tid + i * 256, row = c / CPR, col = (c % CPR) * 8;
-            *reinterpret_cast<half8 *>(&lds[buf][row * PITCH + col]) = stg[i];
-        }
-        if (tid < QT) lse_s[buf][tid] = stg_lse;
-    };
-
-    if (nst > 0) { gload(0, 0); lstore(0); }
-    __syncthreads();
-    int hs = 0, ti = 0;  // head and query tile of stage s, advanced incrementally
-    for (int s = 0; s < nst; ++s) {
-        const int t = t_begin + ti;
-        if (ti == 0) {  // new head: fetch this wave's key fragments
-            const _Float16 *kp = a.k + (int64_t)b * a.ks_b + (int64_t)kv_head(h_begin + hs, a.kv_group, a.kv_magic) * a.ks_h;
-#pragma unroll
-            for (int na = 0; na < NA; ++na) {
-                const _Float16 *row = kp + (int64_t)min(kw0 + na * 32 + r, a.Sk - 1) * a.ks_s + g * 8;
-#pragma unroll
-                for (int tt = 0; tt < NT; ++tt) {
-                    half8 v = load8(row + tt * 16);
-                    kf[na][tt] = a.negate ? flip_sign(v) : v;
-                }
-            }
-        }
-        const int ti1 = (ti + 1 == nt) ? 0 : ti + 1, hs1 = (ti + 1 == nt) ? hs + 1 : hs;
-        if (s + 1 < nst) gload(hs1, ti1);
-        const _Float16 *tile = lds[s & 1];
-
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            half8 bf[NT];
-#pragma unroll
-            for (int tt = 0; tt < NT; ++tt)
-                bf[tt] = *reinterpret_cast<const half8 *>(&tile[(nb * 32 + r) * PITCH + tt * 16 + g * 8]);
-            // p = 2^((s - m) * c - log2 l).  m is 0 unless pass 1 had to stabilise this row; then the
-            // subtraction comes first, so that scores of any magnitude keep their low bits.
-            const float2 st = lse_s[s & 1][nb * 32 + r];
-            const float nlse = -st.y;
-            const bool shifted = __builtin_amdgcn_ballot_w64(st.x != 0.f) != 0;  // wave-uniform
-            const int qmin = t * QT + nb * 32;
-            const bool edge = a.causal && (kmax_w > a.k_past + qmin);  // wave-uniform: straddles the diagonal
-            const int lim = a.k_past + qmin + r;                       // last key this lane's query sees
-            floatx16 cn[NA];
-#pragma unroll
-            for (int na = 0; na < NA; ++na)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) cn[na][i] = 0.f;
-#pragma unroll
-            for (int tt = 0; tt < NT; ++tt)
-#pragma unroll
-                for (int na = 0; na < NA; ++na)
-                    cn[na] = mfma16<BF>(kf[na][tt], bf[tt], cn[na]);
-#pragma unroll
-            for (int na = 0; na < NA; ++na) {
-                if (shifted) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) cn[na][i] -= st.x;
-                }
-                if (!edge) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) colacc[na][i] += fast_exp2(fmaf(cn[na][i], a.c, nlse));
-                } else {
-                    int kb_e = kw0 + na * 32 + 4 * g;  // opaque: keeps the key indices inside this branch
-                    asm volatile("" : "+v"(kb_e));
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const float p = fast_exp2(fmaf(cn[na][i], a.c, nlse));
-                        colacc[na][i] += (kb_e + (8 * (i >> 2) + (i & 3)) <= lim) ? p : 0.f;
-                    }
-                }
-            }
-        }
-
-        if (s + 1 < nst) lstore((s + 1) & 1);
-        __syncthreads();
-        ti = ti1;
-        hs = hs1;
-    }
-
-    // sum the 32 query lanes of each half-wave; lane r == 0 of each half writes its 16 keys
-    const bool direct = (a.gh * a.gq == 1);
-#pragma unroll
-    for (int na = 0; na < NA; ++na) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            float v = colacc[na][i];
-            v += __shfl_xor(v, 16);
-            v += __shfl_xor(v, 8);
-            v += __shfl_xor(v, 4);
-            v += __shfl_xor(v, 2);
-            v += __shfl_xor(v, 1);
-            const int key = kw0 + na * 32 + acc_row(i, g);
-            if (r == 0 && key < a.Sk) {
-                if (direct) {
-                    a.out[(int64_t)b * a.Sk + key] = v * a.inv_norm;
-                    if (a.out_h) a.out_h[(int64_t)b * a.Sk + key] = (_Float16)(v * a.inv_norm);
-                } else
-                    a.partial[((int64_t)grp * a.B + b) * a.Sk + key] = v;
             }
         }
     }

@@ -8,13 +8,11 @@
 namespace fcs {
 
 constexpr int kWavesPerBlock = 4;   // 256 threads
-constexpr int kStageKeys = 64;      // keys staged in LDS per step of the row-statistics pass
-constexpr int kStageRows = 64;      // query rows staged in LDS per step of the column pass
+constexpr int kStageKeys = 64;      // keys staged in LDS per step of either pass
 constexpr int kComputeUnits = 256;  // MI355X
 constexpr int kFusedMaxKeys = 2048; // 8 waves x 8 tiles x 32 keys of fp32 scores per 32 query rows
 constexpr int kFewRowsMaxRows = 4;      // few-rows path: at most this many averaged query rows per head ...
 constexpr int kFewRowsMaxScores = 12288; // ... and rows * Sk scores (48 KB of LDS)
-constexpr int kTargetBlocks = 1024; // 256 CUs x 4: enough workgroups to fill the chip twice over
 
 // column pass (fcs_stream.hip): ring slots of 64-key stages and keys per workgroup chunk, sized so
 // that the LDS ring plus one accumulator slice per wave fit (twice per compute unit for 4-wave blocks)
@@ -33,11 +31,6 @@ struct Plan {
     int n_chunks;    // key-axis splits (partial (max,sum) per chunk when > 1)
     int chunk_keys;  // keys per split, multiple of kStageKeys
     int rows_pad;    // n_qblk * 4 * qw  (row pitch of the statistics arrays)
-    // pass 2: column sums.  grid = (n_kblk, gh*gq, B)
-    int kw;          // keys per wave (32 or 64); a block covers 4*kw keys
-    int n_kblk;
-    int gh, gq;      // groups along heads / along staged query tiles
-    int heads_per_group, qtiles_per_group;
     // column pass: grid = (c_nchunks, c_groups, B); a block owns c_chunk keys and walks over c_upg
     // (head, row block) units
     int c_nb, c_waves; // 32-row fragments per wave, waves per block: a unit has 32 * c_nb * c_waves rows
@@ -56,7 +49,7 @@ struct Plan {
     // workspace layout (byte offsets, each 256-byte aligned)
     size_t off_lse;      // float2 [B*H][rows_pad]            row maximum and log2 of the row sum
     size_t off_ml;       // float2 [B*H][n_chunks][rows_pad]  only when n_chunks > 1
-    size_t off_partial;  // float  [gh*gq][B][Sk]             only when gh*gq > 1
+    size_t off_partial;  // float  [c_groups][B][Sk]          only when c_groups > 1
     size_t total;
 };
 
@@ -90,42 +83,6 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     if (want < 1) want = 1;
     p.chunk_keys = ceil_div(ceil_div(Sk, want), kStageKeys) * kStageKeys;
     p.n_chunks = ceil_div(Sk, p.chunk_keys);
-
-    // ---- pass 2
-    const int n_qt = ceil_div(p.q_rows, kStageRows);
-    p.kw = ((long)ceil_div(Sk, 256) * B >= kTargetBlocks / 4) ? 64 : 32;
-    const int kblk = kWavesPerBlock * p.kw;
-    p.n_kblk = ceil_div(Sk, kblk);
-    // Groups along heads and along staged query tiles, chosen by a small cost model in units of
-    // one stage (64 query rows against the block's keys): a block pays for its stages, for each
-    // head's key fragments, and for starting and finishing; blocks run in generations of as many
-    // as the GPU holds at once (registers allow 4 / 2 blocks per compute unit at D = 64, 3 / 2 at
-    // D = 128 for 32 / 64 keys per wave).
-    const long base2 = (long)p.n_kblk * B;
-    const int per_cu = (p.kw == 64) ? 2 : (D == 64 ? 4 : 3);
-    const long resident = (long)kComputeUnits * per_cu;
-    double best = 0.;
-    p.gh = 1; p.gq = 1; p.heads_per_group = H; p.qtiles_per_group = n_qt;
-    bool first = true;
-    for (int hpg = 1; hpg <= H; hpg = (hpg < 4) ? hpg + 1 : hpg + hpg / 2) {
-        const int gh = ceil_div(H, hpg);
-        const int hpg_e = ceil_div(H, gh);
-        for (int gen = 0; gen <= 2; ++gen) {  // query groups: none, or enough for one / two generations
-            long gq = (gen == 0) ? 1 : (resident * gen + base2 * gh - 1) / (base2 * gh);
-            if (gq > n_qt) gq = n_qt;
-            if (gq < 1) gq = 1;
-            const int tpg = ceil_div(n_qt, (int)gq);
-            const int gq_e = ceil_div(n_qt, tpg);
-            const long blocks = base2 * gh * gq_e;
-            const double gens = (double)((blocks + resident - 1) / resident);
-            const double cost = gens * (hpg_e * (tpg + 1.0) + 3.0) + 0.02 * gh * gq_e;
-            if (first || cost < best) {
-                first = false;
-                best = cost;
-                p.gh = gh; p.heads_per_group = hpg_e; p.gq = gq_e; p.qtiles_per_group = tpg;
-            }
-        }
-    }
 
     // ---- column pass (streaming kernel)
     {

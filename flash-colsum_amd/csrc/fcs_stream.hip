@@ -15,8 +15,8 @@
 //     log2 l_i after it.)
 //   * Summing p over the rows of a tile is in-lane; the two half-waves (which hold different
 //     rows of the same keys) are added with v_permlane32_swap, and the wave adds its total for
-//     the stage's keys into ITS OWN slice of an LDS accumulator with ds_add_f32.  One lane is the
-//     only writer of an address, stage after stage, so the order of additions is fixed.
+//     the stage's keys into ITS OWN slice of an LDS accumulator (plain read-modify-write; a slot has
+//     one writer, stage after stage, so the order of additions is fixed).
 //   * K is streamed: the waves of a workgroup share 64-key stages that they fetch with
 //     global_load_lds_dwordx4 straight into an LDS ring, several stages ahead, XOR-swizzled so
 //     that the operand reads (ds_read_b128, 32 rows a row pitch apart) are conflict-free.  One
@@ -29,6 +29,8 @@
 // unit sees, only stages on the diagonal (or past the last key) take the masked code path.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "fcs_device.h"
 #include "fcs_kernels.h"
@@ -209,12 +211,15 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
 
         // key fragment `na` of the stage in `slot` as MFMA B operand.  Inline assembly: the compiler
         // would make an ordinary LDS read wait for ALL outstanding DMA (vmcnt(0)).
-        auto take_frag = [&](int slot, int na, half8 (&kf)[NT]) {
-            const uint32_t off = (uint32_t)(slot * STAGE_BYTES + na * 32 * ROW_BYTES);
+        // The byte offset of (slot, fragment) is an immediate of the instruction: the stage loop
+        // below is unrolled over the ring so that every slot number is a compile-time constant.
+        auto take_frag = [&](auto off_c, half8 (&kf)[NT]) {
+            constexpr int OFF = decltype(off_c)::value;
+            static_assert(OFF >= 0 && OFF < 65536, "ds_read offset field");
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                const uint32_t ad = take[t] + off;
-                asm volatile("ds_read_b128 %0, %1" : "=v"(kf[t]) : "v"(ad) : "memory");
+                const uint32_t ad = take[t];
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kf[t]) : "v"(ad), "n"(OFF) : "memory");
             }
         };
         auto frag_wait = [&](half8 (&kf)[NT]) {
@@ -257,12 +262,99 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
         // rows of this wave relative to the causal diagonal; non-causal: every key below Sk is visible
         const int kp_eff = a.causal ? a.k_past : 0x3fffffff - a.Sq;
         const int thr_wave_min = a.causal ? min(a.k_past + qw0, a.Sk - 1) : a.Sk - 1;   // last key EVERY row of the wave sees
-        const int thr_wave_max = a.causal ? a.k_past + qw0 + ROWS_W - 1 : 0x3fffffff;  // last key ANY row of the wave sees
 
+        // ---- the stream.  A stage is NA * NB tiles of 32 rows x 32 keys; tile q = na * NB + nb uses key
+        // fragment na and accumulator q & 1.  Software pipeline inside the wave: the MFMA chain of tile q
+        // is issued BEFORE the exponent work of tile q - 1, so the matrix pipe and the VALU run together
+        // whatever the phase of the other wave on the SIMD.
+        constexpr int TILES = NA * NB;
+        static_assert(TILES % 2 == 0, "two accumulators alternate");
         half8 kf[NT];
-        take_frag(0, 0, kf);
-        int slot = 0;
-        for (int st = 0; st < nst; ++st) {
+        take_frag(std::integral_constant<int, 0>{}, kf);
+        floatx16 acc[2];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[0][i] = acc[1][i] = 0.f;
+        float cp[4] = {0.f, 0.f, 0.f, 0.f};  // running column sums of the fragment being exponentiated
+
+        // Exponent work of one finished tile (kb_t: first key of its stage), split in three so that the
+        // common case can be woven between the MFMAs of the next tile:
+        //   drain_begin   requests the fragment's accumulator slot (first row fragment only)
+        //   drain_slow    masked / stabilised forms, all sixteen scores at once
+        //   drain_end     after the last row fragment: fold the half-waves, add into the wave's slice
+        float col_old = 0.f;
+        uint32_t col_ad = 0;
+        auto drain_begin = [&](int kb_t, int na, int nb) {
+            if (nb == 0) {
+                col_ad = lds_addr(colw_w) + (uint32_t)((kb_t - c0 + na * 32 + n) * 4);
+                asm volatile("ds_read_b32 %0, %1" : "=v"(col_old) : "v"(col_ad) : "memory");
+            }
+        };
+        auto drain_slow = [&](const floatx16 &sc, int kb_t, int na, int nb) {
+            const int key = kb_t + na * 32 + n;
+            // visible  <=>  key < Sk  and  key - k_past - (row of register i) <= 0
+            int rel = (key < a.Sk) ? key - kp_eff - (qw0 + 4 * g) : 0x3fffffff;
+            asm volatile("" : "+v"(rel));
+            if (shifted) {
+                // rare: the accumulators started at 0, so the scores carry the very bits pass 1 saw;
+                // m_i is subtracted before the scale and log2 l_i after it
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    floatx4 l4, m4;
+                    const uint32_t ro = (uint32_t)((wave * ROWS_W + nb * 32 + 8 * i4 + 4 * g) * 4);
+                    const uint32_t ad = lds_addr(lg_s) + ro, am = lds_addr(cm_s) + ro;
+                    asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
+                                 : "=&v"(l4), "=&v"(m4)
+                                 : "v"(ad), "v"(am)
+                                 : "memory");
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float pr = fast_exp2(fmaf(sc[4 * i4 + j] + m4[j], cmul, -l4[j]));
+                        cp[j] += (rel <= nb * 32 + 8 * i4 + j) ? pr : 0.f;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float pr = fast_exp2(sc[i] * cmul);
+                    cp[i & 3] += (rel <= nb * 32 + 8 * (i >> 2) + (i & 3)) ? pr : 0.f;
+                }
+            }
+        };
+        auto drain_end = [&](int nb) {
+            if (nb == NB - 1) {
+                float tot = (cp[0] + cp[1]) + (cp[2] + cp[3]);
+                cp[0] = cp[1] = cp[2] = cp[3] = 0.f;
+                // v_permlane32_swap exchanges the upper half of its first operand with the lower half of
+                // its second: started from two copies of the value, one register then holds the lower
+                // half-wave's values in both halves and the other the upper half-wave's, so their sum is
+                // the total of the two half-waves in every lane.  (Inline assembly: given the same value
+                // twice, the builtin's two results were folded into one.)
+                float x = tot, y = tot;
+                asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
+                tot = x + y;
+                // plain read-modify-write of the wave's own slot (LDS float atomics are slow): the old
+                // value was requested before the exponent work; both half-waves store the same total
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(col_old)::"memory");
+                tot += col_old;
+                asm volatile("ds_write_b32 %0, %1" ::"v"(col_ad), "v"(tot) : "memory");
+            }
+        };
+
+        // MFMA chain of one tile alone
+        auto chain = [&](int nb) {
+            floatx16 c = mfma16<BF>(qf[nb][0], kf[0], cinit[nb]);
+#pragma unroll
+            for (int t = 1; t < NT; ++t) c = mfma16<BF>(qf[nb][t], kf[t], c);
+            return c;
+        };
+        auto drain_fast = [&](const floatx16 &sc) {  // every key of the tile visible, no stabilised row
+#pragma unroll
+            for (int i = 0; i < 16; ++i) cp[i & 3] += fast_exp2(sc[i] * cmul);
+        };
+
+        // one stage, in ring slot SLOT (compile-time)
+        auto stage = [&](int st, auto slot_c) {
+            constexpr int SLOT = decltype(slot_c)::value;
             const int kb = c0 + st * KT;
             if (st > 0) {
                 // stage st + 1 has landed (this wave's pieces; the barrier extends that to everyone's), and
@@ -270,96 +362,50 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
                 FCS_WAIT_VM((NS - 3) * IPW);
                 block_barrier();
             }
-            {
-                int free_slot = slot - 1;
-                if (free_slot < 0) free_slot += NS;
-                fetch_stage(st + NS - 1, free_slot);
-            }
-            const bool hidden = kb > thr_wave_max;  // wave-uniform: no row of this wave sees any key of the stage
-            float colt[NA];
+            fetch_stage(st + NS - 1, (SLOT + NS - 1) % NS);
 #pragma unroll
-            for (int na = 0; na < NA; ++na) {
-                floatx16 acc[NB];
-                frag_wait(kf);
-                if (!hidden) {
-#pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) {
-                        acc[nb] = mfma16<BF>(qf[nb][0], kf[0], cinit[nb]);
-#pragma unroll
-                        for (int t = 1; t < NT; ++t) acc[nb] = mfma16<BF>(qf[nb][t], kf[t], acc[nb]);
+            for (int q = 0; q < TILES; ++q) {
+                const int na = q / NB, nb = q % NB;
+                // the previous tile: the one before in this stage, or the last of the previous stage
+                const int p_kb = (q > 0) ? kb : kb - KT;
+                const int p_na = (q > 0) ? (q - 1) / NB : NA - 1, p_nb = (q > 0) ? (q - 1) % NB : NB - 1;
+                const bool have_prev = (q > 0) || (st > 0);
+                const bool p_fast = !shifted && !(p_kb + p_na * 32 + 31 > thr_wave_min);  // wave-uniform
+                auto do_chain = [&]() {
+                    if (nb == 0) frag_wait(kf);
+                    acc[q & 1] = chain(nb);
+                    asm volatile("" : "+v"(acc[0]), "+v"(acc[1]));  // the chain stays where it was written
+                    if (nb == NB - 1) {  // this fragment's last chain has been issued: read back the next one
+                        if (na == 0) take_frag(std::integral_constant<int, SLOT * STAGE_BYTES + 32 * ROW_BYTES>{}, kf);
+                        else take_frag(std::integral_constant<int, ((SLOT + 1) % NS) * STAGE_BYTES>{}, kf);
                     }
-                }
-                // the next fragment is read back while the matrix pipe and the exponents run
-                if (na + 1 < NA) {
-                    take_frag(slot, na + 1, kf);
-                } else {
-                    int nslot = slot + 1;
-                    if (nslot == NS) nslot = 0;
-                    take_frag(nslot, 0, kf);
-                }
-                float cp[4] = {0.f, 0.f, 0.f, 0.f};
-                if (!hidden) {
-                    const int key = kb + na * 32 + n;
-                    const bool edge = kb + na * 32 + 31 > thr_wave_min;  // wave-uniform
-                    if (shifted) {
-                        // rare: the accumulators started at 0, so the scores carry the very bits pass 1 saw;
-                        // m_i is subtracted before the scale and log2 l_i after it
-                        int rel = (key < a.Sk) ? key - kp_eff - (qw0 + 4 * g) : 0x3fffffff;
-#pragma unroll
-                        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                            for (int i4 = 0; i4 < 4; ++i4) {
-                                floatx4 l4, m4;
-                                const uint32_t ro = (uint32_t)((wave * ROWS_W + nb * 32 + 8 * i4 + 4 * g) * 4);
-                                const uint32_t ad = lds_addr(lg_s) + ro, am = lds_addr(cm_s) + ro;
-                                asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
-                                             : "=&v"(l4), "=&v"(m4)
-                                             : "v"(ad), "v"(am)
-                                             : "memory");
-#pragma unroll
-                                for (int j = 0; j < 4; ++j) {
-                                    const float p = fast_exp2(fmaf(acc[nb][4 * i4 + j] + m4[j], cmul, -l4[j]));
-                                    cp[j] += (rel <= nb * 32 + 8 * i4 + j) ? p : 0.f;
-                                }
-                            }
-                    } else if (!edge) {
-#pragma unroll
-                        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                            for (int i = 0; i < 16; ++i) cp[i & 3] += fast_exp2(acc[nb][i] * cmul);
-                    } else {
-                        // visible  <=>  key < Sk  and  key - k_past - (row of register i) <= 0
-                        int rel = (key < a.Sk) ? key - kp_eff - (qw0 + 4 * g) : 0x3fffffff;
-                        asm volatile("" : "+v"(rel));
-#pragma unroll
-                        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                            for (int i = 0; i < 16; ++i) {
-                                const float p = fast_exp2(acc[nb][i] * cmul);
-                                cp[i & 3] += (rel <= nb * 32 + 8 * (i >> 2) + (i & 3)) ? p : 0.f;
-                            }
-                    }
-                }
-                colt[na] = (cp[0] + cp[1]) + (cp[2] + cp[3]);
+                };
+                auto do_drain = [&]() {
+                    if (!have_prev) return;
+                    drain_begin(p_kb, p_na, p_nb);
+                    if (p_fast) drain_fast(acc[(q - 1) & 1]);
+                    else drain_slow(acc[(q - 1) & 1], p_kb, p_na, p_nb);
+                    drain_end(p_nb);
+                    asm volatile("" : "+v"(acc[0]), "+v"(acc[1]));
+                };
+                // Chain first: the matrix pipe works on tile q while the VALU exponentiates tile q - 1.
+                // (Measured slower: the exponent work woven between the chain's MFMAs, and the two waves
+                // of a SIMD in opposite order.)
+                do_chain();
+                do_drain();
             }
-            // the two half-waves hold different rows of the same keys: add them, then the lower half adds
-            // the stage's totals into this wave's slice of the chunk accumulator
-            if (!hidden) {
-#pragma unroll
-                for (int na = 0; na < NA; ++na) {
-                    const int vi = __builtin_bit_cast(int, colt[na]);
-                    const auto sw = __builtin_amdgcn_permlane32_swap(vi, vi, false, false);
-                    const float other = __builtin_bit_cast(float, g == 0 ? sw[1] : sw[0]);
-                    colt[na] += other;
-                }
-                if (g == 0) {
-                    const uint32_t ad = lds_addr(colw_w) + (uint32_t)((kb - c0 + n) * 4);
-                    asm volatile("ds_add_f32 %0, %1" ::"v"(ad), "v"(colt[0]) : "memory");
-                    asm volatile("ds_add_f32 %0, %1 offset:128" ::"v"(ad), "v"(colt[1]) : "memory");
-                }
-            }
-            slot = (slot + 1 == NS) ? 0 : slot + 1;
+        };
+        static_assert(NA == 2, "fragment offsets above");
+        for (int st0 = 0; st0 < nst; st0 += NS) {
+            stage(st0, std::integral_constant<int, 0>{});
+            if (st0 + 1 < nst) stage(st0 + 1, std::integral_constant<int, 1>{});
+            if (st0 + 2 < nst) stage(st0 + 2, std::integral_constant<int, 2>{});
+            if (NS > 3 && st0 + 3 < nst) stage(st0 + 3, std::integral_constant<int, 3 % NS>{});
         }
+        static_assert(NS <= 4, "unrolled above");
+        drain_begin(c0 + (nst - 1) * KT, NA - 1, NB - 1);
+        drain_slow(acc[(TILES - 1) & 1], c0 + (nst - 1) * KT, NA - 1, NB - 1);
+        drain_end(NB - 1);
         // the look-ahead fetches and the operand read-back issued past the last stage must be over before
         // the next unit reuses the ring (and nl_s)
         FCS_WAIT_VM(0);
