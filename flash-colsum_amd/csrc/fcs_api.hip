@@ -56,7 +56,7 @@ int run(int bf16, int causal, const void *q, const void *k, float *out, void *ou
     if (!q || !k || !out || !qs || !ks) return FCS_E_NULL;
     if (B < 1 || H < 1 || Hk < 1 || Sq < 1 || Sk < 1 || D < 1 || cls_n == 0 || k_past < 0) return FCS_E_DIMS;
     if (H % Hk != 0) return FCS_E_DIMS;
-    if (D != 64 && D != 128) return FCS_E_HEAD_DIM;
+    if (D < 8 || D > 256 || (D & 7)) return FCS_E_HEAD_DIM;
     if (!strides_ok(qs, B > 1) || !strides_ok(ks, B > 1) || !aligned16(q) || !aligned16(k)) return FCS_E_STRIDE;
     if (!isfinite(scale)) return FCS_E_SCALE;
 
@@ -75,6 +75,7 @@ int run(int bf16, int causal, const void *q, const void *k, float *out, void *ou
     a.qs_b = qs[0]; a.qs_h = qs[1]; a.qs_s = qs[2];
     a.ks_b = ks[0]; a.ks_h = ks[1]; a.ks_s = ks[2];
     a.B = B; a.H = H; a.Sq = Sq; a.Sk = Sk;
+    a.D = D;
     a.kv_group = H / Hk;
     a.kv_magic = (uint32_t)((0x100000000ull + (uint64_t)a.kv_group - 1) / (uint64_t)a.kv_group);  // unused when the group is 1
     a.q_rows = p.q_rows;
@@ -107,7 +108,7 @@ const char *fcs_strerror(int code)
     case FCS_OK: return "ok";
     case FCS_E_NULL: return "a required pointer is NULL";
     case FCS_E_DIMS: return "invalid dimension (each of B,H,S,D must be >= 1, Hq a multiple of Hk, cls_n != 0, k_past >= 0; B*H <= 65535 on the two-pass path)";
-    case FCS_E_HEAD_DIM: return "unsupported head dim (compiled: 64, 128)";
+    case FCS_E_HEAD_DIM: return "unsupported head dim (a multiple of 8 from 8 to 256)";
     case FCS_E_STRIDE: return "unsupported layout (last stride must be 1; rows, heads and base 16-byte aligned)";
     case FCS_E_WORKSPACE: return "workspace smaller than fcs_workspace_bytes() or not 256-byte aligned";
     case FCS_E_DTYPE: return "unknown operand dtype (FCS_DTYPE_F16 or FCS_DTYPE_BF16)";

@@ -5,12 +5,13 @@
 
 namespace fcs {
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));  // 8 fp16 or (bit pattern) 8 bf16 values
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
+static constexpr half8 kZero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 static constexpr float kNegBig = -1.0e30f;  // "hidden" score: finite so that max/sub never make NaN
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

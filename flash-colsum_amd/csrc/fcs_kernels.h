@@ -13,6 +13,7 @@ struct Args {
     int64_t qs_b, qs_h, qs_s;  // element strides (last dim is 1)
     int64_t ks_b, ks_h, ks_s;
     int B, H, Sq, Sk;
+    int D;               // head dim of the tensors (a multiple of 8); kernels compiled for a wider head read zeros beyond it
     int kv_group;        // query heads per key head (1 unless grouped-query): key head = head / kv_group
     uint32_t kv_magic;   // ceil(2^32 / kv_group), for the division above (unused when kv_group == 1)
     int q_rows;          // query rows that are averaged

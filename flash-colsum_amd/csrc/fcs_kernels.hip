@@ -64,7 +64,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
         const _Float16 *row = qp + (int64_t)min(qi, a.Sq - 1) * a.qs_s + g * 8;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            half8 v = load8(row + t * 16);
+            half8 v = kZero8;  // channels past the tensor's head dim (D is the compiled width) are zeros
+            if (t * 16 + g * 8 < a.D) v = load8(row + t * 16);
             qf[nb][t] = a.negate ? flip_sign(v) : v;
         }
         thr[nb] = a.causal ? min(a.k_past + qi, a.Sk - 1) : a.Sk - 1;
@@ -80,7 +81,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstats_kernel(const Args 
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * THREADS, row = c / CPR, col = (c % CPR) * 8;
-            stg[i] = load8(kp + (int64_t)min(kb + row, a.Sk - 1) * a.ks_s + col);
+            stg[i] = kZero8;
+            if (col < a.D) stg[i] = load8(kp + (int64_t)min(kb + row, a.Sk - 1) * a.ks_s + col);
         }
     };
     auto lstore = [&](int buf) {
@@ -325,12 +327,17 @@ static hipError_t launch_d(const Plan &p, const Args &a, hipStream_t st)
     const dim3 blk(256);
     {
         const dim3 grid(p.n_qblk, p.n_chunks, p.B * p.H);
-        if (p.qw == 64 && p.k1_waves == 8)
-            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64, 8, BF>), grid, dim3(512), 0, st, a);
-        else if (p.qw == 64)
-            hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64, 4, BF>), grid, blk, 0, st, a);
-        else
+        if constexpr (D <= 128) {
+            if (p.qw == 64 && p.k1_waves == 8)
+                hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64, 8, BF>), grid, dim3(512), 0, st, a);
+            else if (p.qw == 64)
+                hipLaunchKernelGGL((fcs_rowstats_kernel<D, 64, 4, BF>), grid, blk, 0, st, a);
+            else
+                hipLaunchKernelGGL((fcs_rowstats_kernel<D, 32, 4, BF>), grid, blk, 0, st, a);
+        } else {  // 64 query rows per wave would not fit the registers
+            if (p.qw != 32 || p.k1_waves != 4) return hipErrorInvalidValue;
             hipLaunchKernelGGL((fcs_rowstats_kernel<D, 32, 4, BF>), grid, blk, 0, st, a);
+        }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -352,9 +359,9 @@ int launch_colsum(const Plan &p, const Args &a, void *stream)
     if (p.fused) return (int)launch_fused(p, a, st);
     hipError_t e;
     if (p.bf16)
-        e = (p.D == 64) ? launch_d<64, true>(p, a, st) : launch_d<128, true>(p, a, st);
+        e = (p.Dp == 64) ? launch_d<64, true>(p, a, st) : (p.Dp == 128) ? launch_d<128, true>(p, a, st) : launch_d<256, true>(p, a, st);
     else
-        e = (p.D == 64) ? launch_d<64, false>(p, a, st) : launch_d<128, false>(p, a, st);
+        e = (p.Dp == 64) ? launch_d<64, false>(p, a, st) : (p.Dp == 128) ? launch_d<128, false>(p, a, st) : launch_d<256, false>(p, a, st);
     return (int)e;
 }
 

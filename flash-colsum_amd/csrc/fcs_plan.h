@@ -16,11 +16,12 @@ constexpr int kFewRowsMaxScores = 12288; // ... and rows * Sk scores (48 KB of L
 
 // column pass (fcs_stream.hip): ring slots of 64-key stages and keys per workgroup chunk, sized so
 // that the LDS ring plus one accumulator slice per wave fit (twice per compute unit for 4-wave blocks)
-constexpr int col_ring_slots(int D, int waves) { return (D >= 128 && waves == 4) ? 3 : 4; }
-constexpr int col_chunk_max(int D, int waves) { return (D >= 128 && waves == 4) ? 1536 : 2048; }
+constexpr int col_ring_slots(int D, int waves) { return (D == 256 || (D == 128 && waves == 4)) ? 3 : 4; }
+constexpr int col_chunk_max(int D, int waves) { return (D == 256) ? 1024 : (D == 128 && waves == 4) ? 1536 : 2048; }
 
 struct Plan {
     int B, H, Sq, Sk, D;
+    int Dp;      // head dim the kernels are compiled for: 64, 128 or 256, the smallest that holds D
     int bf16;    // operands are bf16 instead of fp16 (set by the caller after make_plan)
     int q_rows;  // query rows that are averaged: min(cls_n, Sq) or Sq
     int causal, k_past;
@@ -61,6 +62,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
 {
     if (B < 1 || H < 1 || Sq < 1 || Sk < 1 || D < 1 || k_past < 0) return false;
     p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk; p.D = D;
+    p.Dp = (D <= 64) ? 64 : (D <= 128) ? 128 : 256;
     p.bf16 = 0;
     p.causal = causal ? 1 : 0;
     p.k_past = causal ? k_past : 0;
@@ -69,6 +71,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     // ---- pass 1
     p.qw = (p.q_rows > 128) ? 64 : 32;
     p.k1_waves = (p.q_rows > 256) ? 8 : 4;  // taller blocks re-read the keys less often
+    if (p.Dp == 256) { p.qw = 32; p.k1_waves = 4; }  // the stationary rows of a wider head fill the registers sooner
     const int qblk = p.k1_waves * p.qw;
     p.n_qblk = ceil_div(p.q_rows, qblk);
     p.rows_pad = p.n_qblk * qblk;
@@ -89,10 +92,11 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         if (p.q_rows > 256) { p.c_nb = 2; p.c_waves = 8; }
         else if (p.q_rows > 128) { p.c_nb = 2; p.c_waves = 4; }
         else { p.c_nb = 1; p.c_waves = 4; }
+        if (p.Dp == 256) { p.c_nb = 1; p.c_waves = (p.q_rows > 128) ? 8 : 4; }
         const int block_rows = 32 * p.c_nb * p.c_waves;
         p.c_nrb = ceil_div(p.q_rows, block_rows);
         const long units = (long)H * p.c_nrb;
-        const int chunk_max = col_chunk_max(D, p.c_waves);
+        const int chunk_max = col_chunk_max(p.Dp, p.c_waves);
         const long target = (p.c_waves == 8) ? kComputeUnits : 2 * kComputeUnits;
         int chunk = ceil_div(Sk, kStageKeys) * kStageKeys;
         if (chunk > chunk_max) chunk = chunk_max;
@@ -117,7 +121,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     // ---- few-rows path: a batch of matrix-vector products, one workgroup per (batch entry, head group)
     p.fewrows = 0;
     p.fused = 0;
-    if (!causal && p.q_rows <= kFewRowsMaxRows && (long)p.q_rows * Sk <= kFewRowsMaxScores) {
+    if (!causal && p.q_rows <= kFewRowsMaxRows && (long)p.q_rows * Sk <= kFewRowsMaxScores && (D == 64 || D == 128)) {
         p.fewrows = 1;
         const long bh = (long)B * H;
         int hpb = (int)((bh + 2047) / 2048);  // heads per workgroup: about 2048 workgroups at most

@@ -67,6 +67,9 @@ __device__ __forceinline__ int row_swizzle(int row)
     return D == 64 ? ((row >> 1) & 7) : (row & 15);
 }
 
+// source of the 16-byte pieces that lie past the tensor's head dim (kernels compiled for a wider head)
+__device__ unsigned int g_zero_piece[4];
+
 }  // namespace
 
 template <int D, int NB, int WAVES, bool BF>
@@ -177,9 +180,10 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
                 const _Float16 *row = qp + (int64_t)min(qw0 + nb * 32 + n, a.Sq - 1) * a.qs_s + g * 8;
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    half8 v = load8(row + t * 16);
+                    half8 v = kZero8;  // channels past the tensor's head dim are zeros
+                    if (t * 16 + g * 8 < a.D) v = load8(row + t * 16);
                     if (a.negate) v = flip_sign(v);
-                    if (a.c == 0.f) v = half8{0, 0, 0, 0, 0, 0, 0, 0};
+                    if (a.c == 0.f) v = kZero8;
                     qf[nb][t] = v;
                 }
             }
@@ -193,7 +197,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
         auto fetch_stage = [&](int st, int slot) {
             const int kb = c0 + min(st, nst - 1) * KT;
             char *dst = ring_w + slot * STAGE_BYTES;
-            if (kb + KT <= a.Sk) {  // whole stage inside the tensor (wave-uniform)
+            if (kb + KT <= a.Sk && a.D == D) {  // whole stage inside the tensor, rows as wide as compiled (wave-uniform)
                 const char *src = kp + (int64_t)kb * k_row_b;
 #pragma unroll
                 for (int j = 0; j < IPW; ++j) dma16(src + g_off[j], dst + j * 1024);
@@ -204,7 +208,10 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
                 for (int j = 0; j < IPW; ++j) {
                     const int P = (wave * IPW + j) * 64 + lane_o;
                     const int row = P / PPR, pos = P % PPR;
-                    dma16(kp + (int64_t)min(kb + row, a.Sk - 1) * k_row_b + (pos ^ row_swizzle<D>(row)) * 16, dst + j * 1024);
+                    const int piece = pos ^ row_swizzle<D>(row);
+                    const char *src = kp + (int64_t)min(kb + row, a.Sk - 1) * k_row_b + piece * 16;
+                    if (piece * 8 >= a.D) src = reinterpret_cast<const char *>(g_zero_piece);  // past the head dim: zeros
+                    dma16(src, dst + j * 1024);
                 }
             }
         };
@@ -215,11 +222,11 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
         // below is unrolled over the ring so that every slot number is a compile-time constant.
         auto take_frag = [&](auto off_c, half8 (&kf)[NT]) {
             constexpr int OFF = decltype(off_c)::value;
-            static_assert(OFF >= 0 && OFF < 65536, "ds_read offset field");
+            constexpr int IMM = (OFF < 65536) ? OFF : 0;  // the offset field holds 16 bits
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                const uint32_t ad = take[t];
-                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kf[t]) : "v"(ad), "n"(OFF) : "memory");
+                const uint32_t ad = take[t] + (uint32_t)(OFF - IMM);
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kf[t]) : "v"(ad), "n"(IMM) : "memory");
             }
         };
         auto frag_wait = [&](half8 (&kf)[NT]) {
@@ -444,16 +451,24 @@ static hipError_t launch_cfg(const Plan &p, const Args &a, hipStream_t st)
 template <int D, bool BF>
 static hipError_t launch_colstream_d(const Plan &p, const Args &a, hipStream_t st)
 {
-    if (p.c_nb == 2 && p.c_waves == 8) return launch_cfg<D, 2, 8, BF>(p, a, st);
-    if (p.c_nb == 2 && p.c_waves == 4) return launch_cfg<D, 2, 4, BF>(p, a, st);
-    if (p.c_nb == 1 && p.c_waves == 4) return launch_cfg<D, 1, 4, BF>(p, a, st);
+    if constexpr (D <= 128) {
+        if (p.c_nb == 2 && p.c_waves == 8) return launch_cfg<D, 2, 8, BF>(p, a, st);
+        if (p.c_nb == 2 && p.c_waves == 4) return launch_cfg<D, 2, 4, BF>(p, a, st);
+        if (p.c_nb == 1 && p.c_waves == 4) return launch_cfg<D, 1, 4, BF>(p, a, st);
+    } else {
+        if (p.c_nb == 1 && p.c_waves == 8) return launch_cfg<D, 1, 8, BF>(p, a, st);
+        if (p.c_nb == 1 && p.c_waves == 4) return launch_cfg<D, 1, 4, BF>(p, a, st);
+    }
     return hipErrorInvalidValue;
 }
 
 hipError_t launch_colstream(const Plan &p, const Args &a, hipStream_t st)
 {
-    if (p.bf16) return (p.D == 64) ? launch_colstream_d<64, true>(p, a, st) : launch_colstream_d<128, true>(p, a, st);
-    return (p.D == 64) ? launch_colstream_d<64, false>(p, a, st) : launch_colstream_d<128, false>(p, a, st);
+    if (p.bf16)
+        return (p.Dp == 64) ? launch_colstream_d<64, true>(p, a, st)
+                            : (p.Dp == 128) ? launch_colstream_d<128, true>(p, a, st) : launch_colstream_d<256, true>(p, a, st);
+    return (p.Dp == 64) ? launch_colstream_d<64, false>(p, a, st)
+                        : (p.Dp == 128) ? launch_colstream_d<128, false>(p, a, st) : launch_colstream_d<256, false>(p, a, st);
 }
 
 }  // namespace fcs

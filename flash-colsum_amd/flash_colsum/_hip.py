@@ -22,7 +22,7 @@ _ABI_VERSION = 4
 _lib = None
 
 _I64x4 = ctypes.c_int64 * 4
-_HEAD_DIMS = (64, 128)  # head dims the library is compiled for
+_MAX_HEAD_DIM = 256  # the library takes any multiple of 8 up to this
 
 
 def lib() -> ctypes.CDLL:
@@ -183,11 +183,12 @@ def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n:
         raise ValueError(f"query and key must live on the same GPU, got {q.device} and {k.device}")
     # bf16 inputs run natively when both are bf16; every other dtype is converted to fp16
     dtype = torch.bfloat16 if (q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16) else torch.float16
-    # the kernels are compiled for head dims 64 and 128: smaller ones are padded with zero channels
-    # (a copy), which leaves every score unchanged; the caller's scale already reflects the real D
+    # The library takes head dims that are a multiple of 8 (16-byte rows) up to 256 as they are.  Only a
+    # head dim that is not a multiple of 8 is padded with zero channels to the next one (a copy), which
+    # leaves every score unchanged; the caller's scale already reflects the real D.
     d = q.shape[-1]
-    if d not in _HEAD_DIMS and d < _HEAD_DIMS[-1] and d == k.shape[-1]:
-        pad = next(x for x in _HEAD_DIMS if x > d) - d
+    if d % 8 and d < _MAX_HEAD_DIM and d == k.shape[-1]:
+        pad = 8 - d % 8
         q = torch.nn.functional.pad(q.to(dtype), (0, pad))
         k = torch.nn.functional.pad(k.to(dtype), (0, pad))
     q = _as_kernel_input(q, dtype)

@@ -187,8 +187,8 @@ def test_reference_error_handling():
     with pytest.raises(ValueError, match="same shape"):
         flash_colsum(q, k)
     with pytest.raises(RuntimeError, match="head dim"):
-        flash_colsum(torch.randn(1, 2, 16, 160, device="cuda", dtype=torch.float16),
-                     torch.randn(1, 2, 16, 160, device="cuda", dtype=torch.float16))
+        flash_colsum(torch.randn(1, 2, 16, 320, device="cuda", dtype=torch.float16),
+                     torch.randn(1, 2, 16, 320, device="cuda", dtype=torch.float16))
 
 
 # ---------------------------------------------------------------------------------------
@@ -317,14 +317,39 @@ def test_other_input_dtypes_are_converted_to_fp16():
                   _oracle(q.half().bfloat16().half(), k.half()), "bf16 / fp16 inputs")
 
 
-@pytest.mark.parametrize("d", [8, 32, 40, 80, 96])
-def test_other_head_dims_are_zero_padded(d):
+@pytest.mark.parametrize("d", [8, 32, 40, 80, 96, 160, 192, 256, 20, 100])
+def test_other_head_dims(d):
+    """Head dims other than 64 and 128 run in the kernels compiled for the next of 64 / 128 / 256, which
+    read zeros past the tensor's head dim: no copy when D is a multiple of 8 (20 and 100 are padded to
+    24 and 104 by the host layer, the only copy left)."""
+    from flash_colsum import _hip
+
     q, k = _inputs((2, 3, 150, d), (2, 3, 150, d), seed=7)
     _assert_close(_run(q, k), _oracle(q, k), f"D={d}")
+    _assert_close(_run(q, k, cls_len=2), _oracle(q, k, cls_len=2), f"D={d} cls_len=2")
     q, k = _inputs((1, 3, 50, d), (1, 3, 400, d), seed=8)
     _assert_close(_run(q, k, is_causal=True), _oracle(q, k, is_causal=True), f"causal D={d}")
+    q, k = _inputs((1, 2, 300, d), (1, 2, 2500, d), seed=9)   # 8-wave blocks, several key chunks
+    _assert_close(_run(q, k, is_causal=True, scale=0.05), _oracle(q, k, is_causal=True, scale=0.05), f"causal long D={d}")
+    qb, kb = q.bfloat16(), k.bfloat16()
+    _assert_close(_run(qb, kb, is_causal=True, scale=0.05), _oracle(qb.float(), kb.float(), is_causal=True, scale=0.05),
+                  f"causal long bf16 D={d}")
+    if d % 8 == 0:  # straight through the C ABI, no host-side copy
+        qc, kc = q.cuda(), k.cuda()
+        out = torch.empty((1, 2500), dtype=torch.float32, device="cuda")
+        n_ws = _hip.workspace_bytes(True, 1, 2, 300, 2500, d, -1)
+        ws = torch.empty(max(n_ws, 1), dtype=torch.uint8, device="cuda")
+        rc = _hip.lib().fcs_colsum_causal_f16(qc.data_ptr(), kc.data_ptr(), out.data_ptr(), None, ws.data_ptr(), n_ws, 2, 300, 2500,
+                                              d, 2200, _hip._I64x4(*qc.stride()), _hip._I64x4(*kc.stride()), 0.05,
+                                              torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        _assert_close(out, _oracle(q, k, is_causal=True, scale=0.05), f"C ABI D={d}")
+
+
+def test_head_dims_the_library_rejects():
     with pytest.raises(RuntimeError, match="head dim"):
-        _run(*_inputs((1, 2, 16, 136), (1, 2, 16, 136)))
+        _run(*_inputs((1, 2, 16, 264), (1, 2, 16, 264)))
 
 
 def test_random_shapes_every_path():
@@ -334,7 +359,7 @@ def test_random_shapes_every_path():
 
     rng = random.Random(1234)
     for case in range(60):
-        d = rng.choice([64, 64, 128, 32, 96])
+        d = rng.choice([64, 64, 128, 32, 96, 72, 256])
         h = rng.randint(1, 6)
         mode = rng.choice(["plain", "plain", "cls", "causal"])
         if mode == "causal":

@@ -100,7 +100,7 @@ def test_workspace_plan_over_random_shapes():
         h = rng.choice([1, 2, 8, 16, 32, 40])
         if b * h > 65535:
             continue
-        d = rng.choice([64, 128])
+        d = rng.choice([64, 128, 40, 192, 256])
         sk = rng.choice([1, 5, 64, 577, 2048, 2049, 8191, 65536, 262144])
         sq = rng.choice([1, 16, 128, 512, 1000]) if causal else sk
         cls_n = -1 if causal else rng.choice([-1, 1, 2, 4, 5, 100, sq, sq + 7])
@@ -124,7 +124,8 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert nc(p, p, None, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
     assert nc(p, p, p, None, p, 1 << 30, 0, 8, 16, 64, st, st, 0.125, -1, None) == -2
     assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, 0, None) == -2
-    assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 80, st, st, 0.125, -1, None) == -3
+    assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 84, st, st, 0.125, -1, None) == -3
+    assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 264, st, st, 0.125, -1, None) == -3
     assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 64, bad_last, st, 0.125, -1, None) == -4
     assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 64, st, unaligned, 0.125, -1, None) == -4
     assert nc(ctypes.c_void_p(4098), p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -4
@@ -132,12 +133,12 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert nc(p, p, p, None, None, 0, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
     assert nc(p, p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, float("nan"), -1, None) == -6
     assert ca(p, p, p, None, p, 1 << 30, 8, 16, 64, 64, -1, st, st, 0.125, None) == -2
-    assert ca(p, p, p, None, p, 1 << 30, 8, 16, 64, 96, 48, st, st, 0.125, None) == -3
+    assert ca(p, p, p, None, p, 1 << 30, 8, 16, 64, 4, 48, st, st, 0.125, None) == -3
     assert ca(p, p, p, None, p, 16, 8, 16, 64, 64, 48, st, st, 0.125, None) == -5
     # the bf16 entry points share the checks
     nb, cb = lib.fcs_colsum_noncausal_bf16, lib.fcs_colsum_causal_bf16
     assert nb(None, p, p, None, p, 1 << 30, 2, 8, 16, 64, st, st, 0.125, -1, None) == -1
-    assert nb(p, p, p, None, p, 1 << 30, 2, 8, 16, 80, st, st, 0.125, -1, None) == -3
+    assert nb(p, p, p, None, p, 1 << 30, 2, 8, 16, 81, st, st, 0.125, -1, None) == -3
     assert nb(p, p, p, None, p, 16, 2, 8, 16, 64, st, st, 0.125, -1, None) == -5
     assert cb(p, p, p, None, p, 1 << 30, 8, 16, 64, 64, -1, st, st, 0.125, None) == -2
     assert cb(p, p, p, None, p, 16, 8, 16, 64, 64, 48, st, st, 0.125, None) == -5
