@@ -66,6 +66,12 @@ def lib() -> ctypes.CDLL:
             ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
             ctypes.c_void_p, ctypes.c_size_t] + [ctypes.c_int] * 8 + [
             ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64), ctypes.c_float, ctypes.c_void_p]
+        cdll.fcs_topk_f32.restype = ctypes.c_int
+        cdll.fcs_topk_f32.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                      ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+        cdll.fcs_threshold_f32.restype = ctypes.c_int
+        cdll.fcs_threshold_f32.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_void_p,
+                                           ctypes.c_void_p, ctypes.c_void_p]
         got = cdll.fcs_abi_version()
         if got != _ABI_VERSION:
             raise RuntimeError(f"libflashcolsum.so has ABI {got}, this host layer needs {_ABI_VERSION}")
@@ -236,3 +242,43 @@ def _flash_colsum_causal(Q, K, scale, K_past=None):
     if K_past is None:
         K_past = max(0, K.shape[2] - Q.shape[2])
     return _launch(True, Q, K, scale, -1, int(K_past), want_f16=True)[1]
+
+
+TOPK_SORT_MAX = 4096  # FCS_TOPK_SORT_MAX of include/flash_colsum.h
+
+
+def topk_f32(means: torch.Tensor, k: int, sorted: bool = True):
+    """(values fp32 (B,k), indices int64 (B,k)) of the k largest entries of every row of the fp32 (B,S)
+    means, selected on the GPU on the current stream.  Ties at the k-th value go to the lower index."""
+    if means.dtype != torch.float32 or means.ndim != 2 or means.device.type != "cuda":
+        raise ValueError("means must be a 2-D fp32 GPU tensor")
+    means = means.contiguous()
+    b, s = means.shape
+    idx = torch.empty((b, k), dtype=torch.int64, device=means.device)
+    val = torch.empty((b, k), dtype=torch.float32, device=means.device)
+    in_kernel_sort = sorted and k <= TOPK_SORT_MAX
+    with torch.cuda.device(means.device):
+        stream = torch.cuda.current_stream(means.device).cuda_stream
+        _check(lib().fcs_topk_f32(means.data_ptr(), b, s, int(k), idx.data_ptr(), val.data_ptr(), int(in_kernel_sort), stream),
+               "fcs_topk_f32")
+    if sorted and not in_kernel_sort:
+        # beyond the in-kernel sorting network: a stable sort of the (already index-ordered) selection
+        order = torch.sort(val, dim=1, descending=True, stable=True).indices
+        val, idx = val.gather(1, order), idx.gather(1, order)
+    return val, idx
+
+
+def threshold_f32(means: torch.Tensor, tau: float):
+    """(indices int64 (B,S), counts int32 (B)): row b lists, ascending, the positions whose mean is >= tau
+    in its first counts[b] entries."""
+    if means.dtype != torch.float32 or means.ndim != 2 or means.device.type != "cuda":
+        raise ValueError("means must be a 2-D fp32 GPU tensor")
+    means = means.contiguous()
+    b, s = means.shape
+    idx = torch.empty((b, s), dtype=torch.int64, device=means.device)
+    cnt = torch.empty((b,), dtype=torch.int32, device=means.device)
+    with torch.cuda.device(means.device):
+        stream = torch.cuda.current_stream(means.device).cuda_stream
+        _check(lib().fcs_threshold_f32(means.data_ptr(), b, s, float(tau), idx.data_ptr(), cnt.data_ptr(), stream),
+               "fcs_threshold_f32")
+    return idx, cnt

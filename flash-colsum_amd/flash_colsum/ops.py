@@ -123,4 +123,44 @@ def flash_colsum_ext(
     return _hip.colsum_general(query, key, float(scale), is_causal, cls_n, k_past, want_f16=True)[1]
 
 
-__all__ = ["flash_colsum", "flash_colsum_f32", "flash_colsum_ext"]
+def flash_colsum_topk(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    k: int,
+    scale: Optional[float] = None,
+    is_causal: bool = False,
+    cls_len: Optional[int] = None,
+    sorted: bool = True,
+    extended: bool = False,
+):
+    """The k most-attended key positions of every batch entry: `torch.topk` of the fp32 column means,
+    computed on the GPU right behind them (no fp16 rounding in between, which at long contexts would
+    flush most means to zero; no host synchronisation).
+
+    Returns (values fp32 (B,k), indices int64 (B,k)); `sorted=True` orders them by descending value,
+    `sorted=False` by ascending position.  Ties at the k-th value go to the lower position.
+    `extended=True` accepts the shapes of `flash_colsum_ext`.
+    """
+    if extended:
+        means = flash_colsum_ext(query, key, scale, is_causal, cls_len, out_dtype=torch.float32)
+    else:
+        means = flash_colsum_f32(query, key, scale, is_causal, cls_len)
+    if not 1 <= int(k) <= means.shape[1]:
+        raise ValueError(f"k must be in [1, {means.shape[1]}], got {k}")
+    return _hip.topk_f32(means, int(k), sorted)
+
+
+def flash_colsum_threshold(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    tau: float,
+    scale: Optional[float] = None,
+    is_causal: bool = False,
+    cls_len: Optional[int] = None,
+):
+    """Key positions whose fp32 column mean is >= tau: (indices int64 (B,S), counts int32 (B)); row b
+    lists its positions, ascending, in its first counts[b] entries."""
+    return _hip.threshold_f32(flash_colsum_f32(query, key, scale, is_causal, cls_len), float(tau))
+
+
+__all__ = ["flash_colsum", "flash_colsum_f32", "flash_colsum_ext", "flash_colsum_topk", "flash_colsum_threshold"]

@@ -36,9 +36,9 @@ enum {
     FCS_E_WORKSPACE = -5, /* ws_bytes smaller than fcs_workspace_bytes() for these dims,
                              or ws not 256-byte aligned                                  */
     FCS_E_SCALE = -6,     /* scale is NaN or infinite                                    */
-    FCS_E_DTYPE = -8,     /* fcs_colsum_general: dtype is not FCS_DTYPE_F16 / FCS_DTYPE_BF16 */
-    FCS_E_STATIC_LIMIT = -7 /* fcs_colsum_noncausal_f16_static: the call needs more workspace
-                               than FCS_STATIC_SCRATCH_BYTES                               */
+    FCS_E_STATIC_LIMIT = -7, /* fcs_colsum_noncausal_f16_static: the call needs more workspace
+                                than FCS_STATIC_SCRATCH_BYTES                              */
+    FCS_E_DTYPE = -8      /* fcs_colsum_general: dtype is not FCS_DTYPE_F16 / FCS_DTYPE_BF16 */
 };
 
 /* Size of the per-GPU static scratch array behind fcs_colsum_noncausal_f16_static(). */
@@ -141,6 +141,29 @@ int fcs_colsum_general(int dtype, int causal, const void *q, const void *k, floa
                        void *ws, size_t ws_bytes, int B, int Hq, int Hk, int Sq, int Sk, int D,
                        int cls_n, int k_past, const int64_t q_strides[4], const int64_t k_strides[4],
                        float scale, void *hip_stream);
+
+/* Selection over the fp32 means, for the consumer the reference names (token-importance ranking
+ * for pruning, reference: README.md:10): it runs on the same stream right behind a launch function
+ * above and reads its fp32 `out`, so the small means of long contexts are ranked before the fp16
+ * rounding of the reference's result (reference: flash_colsum/kernel_causal.py:124) can flush them.
+ *
+ * fcs_topk_f32: for every row b of means (B,S) the k largest entries.
+ *   idx_out   (B,k) int64: their positions.  sorted == 0: in ascending position order;
+ *             sorted != 0 (k <= FCS_TOPK_SORT_MAX): by descending value, equal values by ascending
+ *             position.
+ *   val_out   NULL or (B,k) fp32: the values in the same order.
+ *   Ties at the k-th value go to the LOWER position.  Values are compared in the total order of
+ *   their bit patterns (-0 < +0).  Deterministic; needs no workspace.
+ * fcs_threshold_f32: for every row the positions of the entries >= tau, ascending.
+ *   idx_out   (B,S) int64: row b holds count_out[b] positions (the rest is left untouched).
+ *   count_out (B) int32.
+ * Return codes as above (FCS_E_DIMS: k < 1, k > S, or sorted with k > FCS_TOPK_SORT_MAX;
+ * FCS_E_SCALE: tau is NaN). */
+#define FCS_TOPK_SORT_MAX 4096
+int fcs_topk_f32(const float *means, int B, int S, int k, int64_t *idx_out, float *val_out, int sorted,
+                 void *hip_stream);
+int fcs_threshold_f32(const float *means, int B, int S, float tau, int64_t *idx_out, int32_t *count_out,
+                      void *hip_stream);
 
 #ifdef __cplusplus
 }

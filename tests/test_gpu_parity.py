@@ -591,6 +591,93 @@ def test_ext_equals_the_reference_entry_points_bit_for_bit():
 
 
 # ---------------------------------------------------------------------------------------
+# top-k / threshold selection over the fp32 means
+# ---------------------------------------------------------------------------------------
+def _topk_reference(row, k):
+    """k largest by (value descending, index ascending): the tie rule the library states."""
+    order = sorted(range(len(row)), key=lambda i: (-row[i], i))[:k]
+    return order
+
+
+@pytest.mark.parametrize("b,s,k", [(1, 1, 1), (3, 37, 5), (2, 1000, 1), (2, 1000, 1000), (4, 5000, 300), (1, 70000, 4096),
+                                   (2, 3000, 2999), (1, 262144, 5000)])
+def test_topk_kernel_bit_exact(b, s, k):
+    from flash_colsum import _hip
+
+    g = torch.Generator().manual_seed(b * 7 + s + k)
+    x = torch.rand((b, s), generator=g, dtype=torch.float32)
+    # plenty of exact ties, some zeros, some negatives and a run of equal values across the k-th place
+    x[:, ::7] = x[:, min(3, s - 1):min(3, s - 1) + 1].clone()
+    x[:, 2::13] *= -1.0
+    x[:, 5::11] = 0.0   # after the sign flips: the library orders -0 below +0, python's sort does not
+    val, idx = _hip.topk_f32(x.cuda(), k, sorted=True)
+    uval, uidx = _hip.topk_f32(x.cuda(), k, sorted=False)
+    torch.cuda.synchronize()
+    for r in range(b):
+        want = _topk_reference(x[r].tolist(), k)
+        assert idx[r].tolist() == want, (b, s, k, r)
+        assert torch.equal(val[r].cpu(), x[r, want])
+        assert uidx[r].tolist() == sorted(want)
+        assert torch.equal(uval[r].cpu(), x[r, sorted(want)])
+    # the same values as torch.topk picks (its tie order is unspecified, the values are not)
+    assert torch.equal(val.cpu(), torch.topk(x, k, dim=1).values)
+
+
+def test_threshold_kernel_bit_exact():
+    from flash_colsum import _hip
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.rand((3, 4097), generator=g, dtype=torch.float32)
+    x[:, ::5] = 0.25
+    for tau in (0.25, 0.0, 0.999, 2.0, -1.0):
+        idx, cnt = _hip.threshold_f32(x.cuda(), tau)
+        torch.cuda.synchronize()
+        for r in range(3):
+            want = (x[r] >= tau).nonzero().view(-1)
+            assert cnt[r].item() == want.numel(), (tau, r)
+            assert torch.equal(idx[r, : want.numel()].cpu(), want)
+
+
+@pytest.mark.parametrize("qs,ks,kw,k", [
+    ((2, 8, 577, 64), (2, 8, 577, 64), {}, 64),
+    ((1, 16, 128, 128), (1, 16, 16384, 128), {"is_causal": True}, 1024),
+    ((3, 4, 300, 64), (3, 4, 300, 64), {"cls_len": 1}, 30),
+])
+def test_flash_colsum_topk_matches_topk_of_the_oracle(qs, ks, kw, k):
+    """Indices must be those of torch.topk on the float64 oracle wherever the oracle's values are separated
+    by more than the kernels' fp32 error; every index the two disagree on must sit in a near-tie at the
+    k-th place.  At K_len = 16384 most means lie below fp16's normal range: the fp16 result of the
+    reference operator cannot rank them, the fp32 means do."""
+    from flash_colsum import flash_colsum, flash_colsum_topk
+
+    q, k_ = _inputs(qs, ks, seed=23)
+    ref = _oracle(q, k_, **kw)
+    val, idx = flash_colsum_topk(q.cuda(), k_.cuda(), k, **kw)
+    torch.cuda.synchronize()
+    assert val.shape == (qs[0], k) and idx.dtype == torch.int64
+    for r in range(qs[0]):
+        want = torch.topk(ref[r], k).indices
+        got = idx[r].cpu()
+        kth = ref[r, want[-1]].item()
+        differ = set(got.tolist()) ^ set(want.tolist())
+        for j in differ:
+            assert abs(ref[r, j].item() - kth) <= 2e-6 * kth, (r, j, ref[r, j].item(), kth)
+        # descending values, and the values are the fp32 means at those positions
+        assert (val[r, 1:] <= val[r, :-1]).all()
+        _assert_close(val[r].cpu(), ref[r, got], f"top-k values row {r}")
+    if kw.get("is_causal"):
+        half = flash_colsum(q.cuda(), k_.cuda(), **kw)
+        assert (half == 0).float().mean().item() < 0.5  # (informational: fp16 keeps these; smaller means would flush)
+    idx_t, cnt = __import__("flash_colsum").flash_colsum_threshold(q.cuda(), k_.cuda(), float(ref.mean()), **kw)
+    torch.cuda.synchronize()
+    for r in range(qs[0]):
+        want = (ref[r] >= float(ref.mean())).nonzero().view(-1)
+        got = idx_t[r, : cnt[r].item()].cpu()
+        for j in set(got.tolist()) ^ set(want.tolist()):
+            assert abs(ref[r, j].item() - float(ref.mean())) <= 2e-6 * float(ref.mean())
+
+
+# ---------------------------------------------------------------------------------------
 # large score magnitudes: |scale * s| * log2(e) in the thousands
 # ---------------------------------------------------------------------------------------
 @pytest.mark.parametrize("qs,ks,kw,bf16", [

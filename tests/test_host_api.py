@@ -62,8 +62,8 @@ def test_library_exports_every_declared_symbol():
     lib = _hip.lib()
     names = _declared_symbols()
     assert set(names) >= {"fcs_abi_version", "fcs_colsum_causal_bf16", "fcs_colsum_causal_f16", "fcs_colsum_noncausal_bf16",
-                          "fcs_colsum_noncausal_f16", "fcs_colsum_noncausal_f16_static", "fcs_strerror",
-                          "fcs_workspace_bytes"}
+                          "fcs_colsum_noncausal_f16", "fcs_colsum_noncausal_f16_static", "fcs_colsum_general",
+                          "fcs_topk_f32", "fcs_threshold_f32", "fcs_strerror", "fcs_workspace_bytes"}
     for n in names:
         assert getattr(lib, n) is not None
     assert lib.fcs_abi_version() == 4
@@ -142,6 +142,20 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert nb(p, p, p, None, p, 16, 2, 8, 16, 64, st, st, 0.125, -1, None) == -5
     assert cb(p, p, p, None, p, 1 << 30, 8, 16, 64, 64, -1, st, st, 0.125, None) == -2
     assert cb(p, p, p, None, p, 16, 8, 16, 64, 64, 48, st, st, 0.125, None) == -5
+
+
+def test_topk_argument_errors_without_a_gpu():
+    lib = _hip.lib()
+    p = ctypes.c_void_p(4096)
+    assert lib.fcs_topk_f32(None, 1, 8, 2, p, None, 0, None) == -1
+    assert lib.fcs_topk_f32(p, 1, 8, 0, p, None, 0, None) == -2
+    assert lib.fcs_topk_f32(p, 1, 8, 9, p, None, 0, None) == -2
+    assert lib.fcs_topk_f32(p, 1, 100000, _hip.TOPK_SORT_MAX + 1, p, None, 1, None) == -2
+    assert lib.fcs_threshold_f32(p, 1, 8, 0.5, p, None, None) == -1
+    assert lib.fcs_threshold_f32(p, 0, 8, 0.5, p, p, None) == -2
+    assert lib.fcs_threshold_f32(p, 1, 8, float("nan"), p, p, None) == -6
+    text = open(os.path.join(ROOT, "include", "flash_colsum.h")).read()
+    assert f"#define FCS_TOPK_SORT_MAX {_hip.TOPK_SORT_MAX}" in text
 
 
 def test_missing_library_is_loud(monkeypatch, tmp_path):
