@@ -8,7 +8,10 @@ else goes to stderr.
 
   value          effective TFLOP/s of the whole call (wall clock, launch + epilogue
                  included), counting two QK^T passes: 4*B*H*Sq*Sk*D / t
-  ms_per_step    wall-clock milliseconds per call
+  ms_per_step    wall-clock milliseconds per call, calls issued back to back
+  ms_per_call_synced / value_synced
+                 the same with a device synchronize after every call, the reference benchmark's
+                 own clock (reference: benchmarks/benchmark_colsum.py:42-56)
   roofline       kernels-only time of one call (HIP events on the launch stream around the
                  C-ABI call with output and workspace preallocated) against the dense
                  fp16 MFMA peak
@@ -94,6 +97,18 @@ def hbm_bound(name):
     return needed_rows(name) * 16 <= WORKLOADS[name][0][2] and needed_rows(name) <= 16
 
 
+def kernel_source_sha16():
+    """First 16 hex digits of the SHA-256 over the library's kernel sources, in name order."""
+    import hashlib
+
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "flash-colsum_amd", "csrc")
+    for fn in sorted(os.listdir(src)):
+        with open(os.path.join(src, fn), "rb") as f:
+            h.update(fn.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -101,6 +116,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the benchmark line: run the reference's three sweeps (bench_sweep.py) and write "
+                         "their summary as CSV to --sweep-out")
+    ap.add_argument("--sweep-out", default=os.path.join(ROOT, "gpurun_out", "sweeps_mi355x.csv"))
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy five times, so that a rocprofv3 --pmc run over this "
                          "command sees a kernel of known HBM traffic next to the workload's kernels")
@@ -113,6 +132,15 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+    if args.sweep:
+        import bench_sweep
+
+        os.makedirs(os.path.dirname(args.sweep_out), exist_ok=True)
+        sys.argv = ["bench_sweep.py", "--sweep", "all", "--out", args.sweep_out, "--iters", str(max(3, min(args.steps, 50))),
+                    "--warmup", str(max(1, min(args.warmup, 10)))]
+        bench_sweep.main()
+        print(json.dumps({"sweep_csv": args.sweep_out}), flush=True)
+        return
     name = args.workload
     q32, k32, kwargs = make_inputs(name)
     q = q32.half().cuda()
@@ -133,6 +161,12 @@ def main():
     ms_call = (time.perf_counter() - t0) * 1e3 / args.steps
     fl = flops(name)
     tflops = fl / (ms_call * 1e-3) / 1e12
+    # the reference's own clock (benchmarks/benchmark_colsum.py:42-56): call + synchronize per iteration
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        flash_colsum(q, k, **kwargs)
+        torch.cuda.synchronize()
+    ms_call_synced = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # ---- kernels only: HIP events on the launch stream around the C-ABI call
     b, h, sq, d = q.shape
@@ -194,7 +228,8 @@ def main():
         roofline.update({"bound": "hbm", "achieved": round(ker_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": round(ker_gbs / PEAK_HBM_GBS, 4),
                          "needed_tflops": round(fl * needed_rows(name) / q.shape[2] / (ker_ms * 1e-3) / 1e12, 3)})
-    print(f"[bench] {name}: {ms_call:.4f} ms/call wall, {raw_ms:.4f} ms C-ABI back-to-back, {ker_ms:.4f} ms kernels, "
+    print(f"[bench] {name}: {ms_call:.4f} ms/call wall ({ms_call_synced:.4f} with a synchronize per call), "
+          f"{raw_ms:.4f} ms C-ABI back-to-back, {ker_ms:.4f} ms kernels, "
           f"{tflops:.1f} / {ker_tflops:.1f} TFLOP/s", file=sys.stderr)
 
     if args.copy_calibration:
@@ -204,11 +239,16 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
 
-    # measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), bytes per call
+    # measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), bytes per call; only
+    # valid for the kernels it was measured with: the file names the hash of the kernel sources
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(traffic_file):
         with open(traffic_file) as f:
-            roofline["traffic"] = json.load(f).get(name)
+            measured = json.load(f)
+        if measured.get("kernel_source_sha16") == kernel_source_sha16():
+            roofline["traffic"] = measured.get(name)
+        else:
+            roofline["traffic_note"] = "profiles/hbm_traffic.json was measured with other kernel sources: ignored"
 
     # ---- CPU baseline: eager materialising path on the host cores, same workload
     cpu = None
@@ -243,6 +283,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_call, 5),
+        "ms_per_call_synced": round(ms_call_synced, 5),
+        "value_synced": round(fl / (ms_call_synced * 1e-3) / 1e12, 2),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

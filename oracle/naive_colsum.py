@@ -67,7 +67,7 @@ def colsum_exact(
     The score matrix of one row block is (row_block, S_k), so memory stays bounded at the
     largest benchmark shapes.  Scores are computed in the input dtype's float32 upcast
     (exact products of fp16 values, fp32 BLAS accumulation) and the softmax and the
-    running column sums in `acc_dtype`.
+    running column sums in `acc_dtype`.  The result lives on the inputs' device.
     """
     b_n, h_n, s_q, d = query.shape
     s_k = key.shape[2]
@@ -79,8 +79,9 @@ def colsum_exact(
             raise ValueError(f"cls_len must be positive, got {cls_len}")
         rows = min(int(cls_len), s_q)
     k_past = max(0, s_k - s_q)
-    out = torch.zeros(b_n, s_k, dtype=acc_dtype)
-    j = torch.arange(s_k).view(1, s_k)
+    dev = query.device  # runs wherever its inputs live (the tests use a GPU for the longest shapes)
+    out = torch.zeros(b_n, s_k, dtype=acc_dtype, device=dev)
+    j = torch.arange(s_k, device=dev).view(1, s_k)
     for b in range(b_n):
         for h in range(h_n):
             kt = key[b, h].to(torch.float32).t().contiguous()
@@ -88,7 +89,7 @@ def colsum_exact(
                 r1 = min(rows, r0 + row_block)
                 s = (query[b, h, r0:r1].to(torch.float32) @ kt).to(acc_dtype) * scale
                 if is_causal:
-                    i = torch.arange(r0, r1).view(-1, 1)
+                    i = torch.arange(r0, r1, device=dev).view(-1, 1)
                     s = s.masked_fill(j > (i + k_past), float("-inf"))
                 out[b] += torch.softmax(s, dim=-1).sum(dim=0)
     return out / (h_n * rows)
@@ -129,8 +130,9 @@ def colsum_ext_exact(
         rows = min(int(cls_len), s_q)
     if k_past is None:
         k_past = max(0, s_k - s_q)
-    out = torch.zeros(b_n, s_k, dtype=acc_dtype)
-    j = torch.arange(s_k).view(1, s_k)
+    dev = query.device
+    out = torch.zeros(b_n, s_k, dtype=acc_dtype, device=dev)
+    j = torch.arange(s_k, device=dev).view(1, s_k)
     for b in range(b_n):
         for h in range(h_q):
             kt = key[b, h // grp].to(torch.float32).t().contiguous()
@@ -138,7 +140,7 @@ def colsum_ext_exact(
                 r1 = min(rows, r0 + row_block)
                 s = (query[b, h, r0:r1].to(torch.float32) @ kt).to(acc_dtype) * scale
                 if is_causal:
-                    i = torch.arange(r0, r1).view(-1, 1)
+                    i = torch.arange(r0, r1, device=dev).view(-1, 1)
                     s = s.masked_fill(j > (i + k_past), float("-inf"))
                 out[b] += torch.softmax(s, dim=-1).sum(dim=0)
     return out / (h_q * rows)

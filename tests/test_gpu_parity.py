@@ -722,6 +722,31 @@ def test_large_score_magnitudes(qs, ks, kw, bf16):
 
 
 # ---------------------------------------------------------------------------------------
+# one long point of each benchmark sweep (reference: benchmarks/benchmark_colsum.py:757-801)
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("qs,ks,kw", [
+    ((1, 16, 32768, 64), (1, 16, 32768, 64), {}),                       # non-causal B = 1 sweep
+    ((1, 32, 128, 128), (1, 32, 262144, 128), {"is_causal": True}),     # causal sweep, longest point
+    ((256, 16, 1024, 64), (256, 16, 1024, 64), {}),                     # batched sweep
+])
+def test_long_sweep_points(qs, ks, kw):
+    """Both bounds against the float64 oracle at sizes the CPU would need minutes for: the oracle
+    (same code, row-blocked float64 softmax) runs on the GPU here, after a check that it gives the
+    same numbers there as on the CPU at a small shape."""
+    from oracle import colsum_exact
+
+    qsmall, ksmall = _inputs((2, 3, 200, 64), (2, 3, 200, 64), seed=51)
+    assert torch.allclose(colsum_exact(qsmall.cuda(), ksmall.cuda()).cpu(), colsum_exact(qsmall, ksmall), rtol=2e-6, atol=0)  # fp32 BLAS rounding
+    g = torch.Generator(device="cuda").manual_seed(52)
+    q = torch.randn(qs, generator=g, device="cuda", dtype=torch.float16)
+    k = torch.randn(ks, generator=g, device="cuda", dtype=torch.float16)
+    out = _run(q, k, **kw)
+    ref = colsum_exact(q, k, row_block=2048, **kw)
+    _assert_close(out, ref, f"sweep point {qs} {ks}")
+    assert torch.allclose(out.double().sum(-1), torch.ones(qs[0], dtype=torch.float64, device="cuda"), atol=2e-5)
+
+
+# ---------------------------------------------------------------------------------------
 # size-independent properties at the full benchmark sizes
 # ---------------------------------------------------------------------------------------
 def test_full_size_properties():
