@@ -47,7 +47,8 @@ hipError_t launch_fused(const Plan &p, const Args &a, hipStream_t st);
 // few-rows path (fcs_fewrows.hip): p.fewrows == 1
 hipError_t launch_fewrows(const Plan &p, const Args &a, hipStream_t st);
 
-// column pass of the two-pass path (fcs_stream.hip)
+// row-statistics pass and column pass of the two-pass path (fcs_stream.hip)
+hipError_t launch_rowstream(const Plan &p, const Args &a, hipStream_t st);
 hipError_t launch_colstream(const Plan &p, const Args &a, hipStream_t st);
 
 // shared final reduction out = inv_norm * sum of the n_partials slabs (fcs_kernels.hip)

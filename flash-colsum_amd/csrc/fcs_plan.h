@@ -19,6 +19,9 @@ constexpr int kFewRowsMaxScores = 12288; // ... and rows * Sk scores (48 KB of L
 constexpr int col_ring_slots(int D, int waves) { return (D == 256 || (D == 128 && waves == 4)) ? 3 : 4; }
 constexpr int col_chunk_max(int D, int waves) { return (D == 256) ? 1024 : (D == 128 && waves == 4) ? 1536 : 2048; }
 
+// row-statistics pass on the same stream (fcs_stream.hip): ring slots
+constexpr int row_ring_slots(int D, int waves) { return (D == 256 || (D == 128 && waves == 4)) ? 3 : 4; }
+
 struct Plan {
     int B, H, Sq, Sk, D;
     int Dp;      // head dim the kernels are compiled for: 64, 128 or 256, the smallest that holds D

@@ -438,6 +438,293 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
 }
 
 // ------------------------------------------------------------------------------------
+// pass 1 on the same machinery: row maximum and sum of exponentials of one (row block, head, key split)
+// ------------------------------------------------------------------------------------
+// Same orientation and stream as the column pass (Q stationary, K through the LDS-DMA ring), but the
+// exponentials are added up per ROW: register i of a lane keeps the running sum of its row over the
+// lane's keys for the whole split, and the 32 key lanes are added once at the end through LDS.
+// Common case: 2^(c * s) without max subtraction, exact while every row sum of the split stays inside
+// [2^-80, 2^120); a block that leaves that range redoes its keys in two more sweeps (row maxima, then
+// sums of 2^((s - m) * c), the maximum subtracted before the scale).  Writes (m, log2 l) per row, or
+// (m, l) per (split, row) when the keys are split; the column pass merges the splits.
+template <int D, int NB, int WAVES, bool BF>
+__global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args a)
+{
+    constexpr int THREADS = 64 * WAVES;
+    constexpr int NT = D / 16;
+    constexpr int KT = kStageKeys;
+    constexpr int NA = KT / 32;
+    constexpr int ROWS_W = 32 * NB;
+    constexpr int BLOCK_ROWS = WAVES * ROWS_W;
+    constexpr int ROW_BYTES = D * 2;
+    constexpr int PPR = D / 8;
+    constexpr int STAGE_BYTES = KT * ROW_BYTES;
+    constexpr int IPW = KT * PPR / THREADS;
+    constexpr int NS = row_ring_slots(D, WAVES);
+    constexpr int RP = 33;  // floats per row of the transpose buffer
+    static_assert(IPW >= 1 && KT * PPR == IPW * THREADS, "a stage is a whole number of DMA instructions per wave");
+    static_assert(NS >= 3 && NS <= 4, "ring depth");
+    __shared__ __attribute__((aligned(16))) char ring[NS * STAGE_BYTES];
+    __shared__ __attribute__((aligned(16))) float red[WAVES * 32 * RP];  // wave-private [32 rows][RP]
+    __shared__ __attribute__((aligned(16))) float mrow[BLOCK_ROWS];      // row maxima of the stabilised sweeps
+    __shared__ int bad_s[WAVES];
+
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int bx, chunk, bh;  // row blocks of one (key split, head) read the same keys: same XCD
+    xcd_contiguous_block(bx, chunk, bh);
+    const int b = bh / a.H, h = bh - b * a.H;
+    const int row0 = bx * BLOCK_ROWS, qw0 = row0 + wave * ROWS_W;
+    const float cmul = a.c;
+
+    // key range of this block: its split, cut at the last key any of its rows may see
+    const int kc0 = chunk * a.chunk_keys;
+    int kc1 = min(a.Sk, kc0 + a.chunk_keys);
+    if (a.causal) kc1 = min(kc1, a.k_past + min(row0 + BLOCK_ROWS, a.q_rows));
+    const int nst = (kc1 > kc0) ? (kc1 - kc0 + KT - 1) / KT : 0;
+
+    uint32_t g_off[IPW];
+#pragma unroll
+    for (int j = 0; j < IPW; ++j) {
+        const int P = (wave * IPW + j) * 64 + lane;
+        const int row = P / PPR, pos = P % PPR;
+        g_off[j] = (uint32_t)row * (uint32_t)(a.ks_s * 2) + (uint32_t)((pos ^ row_swizzle<D>(row)) * 16);
+    }
+    char *ring_w = ring + wave * (IPW * 1024);
+    uint32_t take[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+        take[t] = lds_addr(ring) + (uint32_t)(n * ROW_BYTES + (((2 * t + g) ^ row_swizzle<D>(n)) * 16));
+
+    half8 qf[NB][NT];
+    {
+        const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const _Float16 *row = qp + (int64_t)min(qw0 + nb * 32 + n, a.Sq - 1) * a.qs_s + g * 8;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                half8 v = kZero8;
+                if (t * 16 + g * 8 < a.D) v = load8(row + t * 16);
+                qf[nb][t] = a.negate ? flip_sign(v) : v;
+            }
+        }
+    }
+    const char *kp = reinterpret_cast<const char *>(a.k + (int64_t)b * a.ks_b +
+                                                    (int64_t)kv_head(h, a.kv_group, a.kv_magic) * a.ks_h);
+    const int64_t k_row_b = a.ks_s * 2;
+    const int kp_eff = a.causal ? a.k_past : 0x3fffffff - a.Sq;
+    const int thr_wave_min = a.causal ? min(a.k_past + qw0, a.Sk - 1) : a.Sk - 1;
+
+    auto fetch_stage = [&](int st, int slot) {
+        const int kb = kc0 + min(st, nst - 1) * KT;
+        char *dst = ring_w + slot * STAGE_BYTES;
+        if (kb + KT <= a.Sk && a.D == D) {
+            const char *src = kp + (int64_t)kb * k_row_b;
+#pragma unroll
+            for (int j = 0; j < IPW; ++j) dma16(src + g_off[j], dst + j * 1024);
+        } else {
+            int lane_o = lane;
+            asm volatile("" : "+v"(lane_o));
+#pragma unroll
+            for (int j = 0; j < IPW; ++j) {
+                const int P = (wave * IPW + j) * 64 + lane_o;
+                const int row = P / PPR, pos = P % PPR;
+                const int piece = pos ^ row_swizzle<D>(row);
+                const char *src = kp + (int64_t)min(kb + row, a.Sk - 1) * k_row_b + piece * 16;
+                if (piece * 8 >= a.D) src = reinterpret_cast<const char *>(g_zero_piece);
+                dma16(src, dst + j * 1024);
+            }
+        }
+    };
+    half8 kf[NT];
+    auto take_frag = [&](auto off_c, half8 (&dst)[NT]) {
+        constexpr int OFF = decltype(off_c)::value;
+        constexpr int IMM = (OFF < 65536) ? OFF : 0;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const uint32_t ad = take[t] + (uint32_t)(OFF - IMM);
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst[t]) : "v"(ad), "n"(IMM) : "memory");
+        }
+    };
+    auto frag_wait = [&](half8 (&dst)[NT]) {
+#pragma unroll
+        for (int t0 = 0; t0 < NT; t0 += 4)
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(dst[t0]), "+v"(dst[t0 + 1]), "+v"(dst[t0 + 2]), "+v"(dst[t0 + 3])::"memory");
+    };
+
+    float rs[NB][16];      // running per-row value (sum or maximum) over this lane's keys
+    float nmax[NB][16];    // -m_i of the rows in accumulator layout (stabilised sum sweep only)
+
+    // One sweep over the block's keys.  MAXOP: rs = max of the visible scores; else rs += 2^(score * c)
+    // over the visible keys.  SHIFT: the row's -m_i (in `nmax`) is added to the score before the scale.  The
+    // accumulators always start at 0, so that every sweep, and the column pass for these rows, sees the
+    // very same score bits.
+    auto sweep = [&](auto max_c, auto shift_c) {
+        constexpr bool MAXOP = decltype(max_c)::value;
+        constexpr bool SHIFT = decltype(shift_c)::value;
+        constexpr int TILES = NA * NB;
+        static_assert(NA == 2 && TILES % 2 == 0, "fragment offsets and the two alternating accumulators");
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) rs[nb][i] = MAXOP ? kNegBig : 0.f;
+        if (nst == 0) return;  // block-uniform
+#pragma unroll
+        for (int st = 0; st < NS - 1; ++st) fetch_stage(st, st);
+        FCS_WAIT_VM((NS - 3) * IPW);
+        block_sync();
+        take_frag(std::integral_constant<int, 0>{}, kf);
+        floatx16 acc[2];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[0][i] = acc[1][i] = 0.f;
+        auto drain = [&](const floatx16 &sc, int kb_t, int na, int nb) {
+            const bool edge = kb_t + na * 32 + 31 > thr_wave_min;  // wave-uniform
+            if (!edge) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    if (MAXOP) rs[nb][i] = fmaxf(rs[nb][i], sc[i]);
+                    else rs[nb][i] += fast_exp2((SHIFT ? sc[i] + nmax[nb][i] : sc[i]) * cmul);
+                }
+            } else {
+                const int key = kb_t + na * 32 + n;
+                int rel = (key < a.Sk) ? key - kp_eff - (qw0 + 4 * g) : 0x3fffffff;
+                asm volatile("" : "+v"(rel));
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const bool vis = rel <= nb * 32 + 8 * (i >> 2) + (i & 3);
+                    if (MAXOP) rs[nb][i] = fmaxf(rs[nb][i], vis ? sc[i] : kNegBig);
+                    else rs[nb][i] += vis ? fast_exp2((SHIFT ? sc[i] + nmax[nb][i] : sc[i]) * cmul) : 0.f;
+                }
+            }
+        };
+        auto stage = [&](int st, auto slot_c) {
+            constexpr int SLOT = decltype(slot_c)::value;
+            const int kb = kc0 + st * KT;
+            if (st > 0) {
+                FCS_WAIT_VM((NS - 3) * IPW);
+                block_barrier();
+            }
+            fetch_stage(st + NS - 1, (SLOT + NS - 1) % NS);
+#pragma unroll
+            for (int q = 0; q < TILES; ++q) {
+                const int na = q / NB, nb = q % NB;
+                if (nb == 0) frag_wait(kf);
+                const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                floatx16 c = mfma16<BF>(qf[nb][0], kf[0], zero16);
+#pragma unroll
+                for (int t = 1; t < NT; ++t) c = mfma16<BF>(qf[nb][t], kf[t], c);
+                acc[q & 1] = c;
+                asm volatile("" : "+v"(acc[0]), "+v"(acc[1]));
+                if (nb == NB - 1) {
+                    if (na == 0) take_frag(std::integral_constant<int, SLOT * STAGE_BYTES + 32 * ROW_BYTES>{}, kf);
+                    else take_frag(std::integral_constant<int, ((SLOT + 1) % NS) * STAGE_BYTES>{}, kf);
+                }
+                if (q > 0) drain(acc[(q - 1) & 1], kb, (q - 1) / NB, (q - 1) % NB);
+                else if (st > 0) drain(acc[(TILES - 1) & 1], kb - KT, NA - 1, NB - 1);
+            }
+        };
+        for (int st0 = 0; st0 < nst; st0 += NS) {
+            stage(st0, std::integral_constant<int, 0>{});
+            if (st0 + 1 < nst) stage(st0 + 1, std::integral_constant<int, 1>{});
+            if (st0 + 2 < nst) stage(st0 + 2, std::integral_constant<int, 2>{});
+            if (NS > 3 && st0 + 3 < nst) stage(st0 + 3, std::integral_constant<int, 3 % NS>{});
+        }
+        drain(acc[(TILES - 1) & 1], kc0 + (nst - 1) * KT, NA - 1, NB - 1);
+        FCS_WAIT_VM(0);
+        frag_wait(kf);
+        block_sync();  // the ring may be refilled by the next sweep
+    };
+
+    // rs[nb][*] over the 32 key lanes: every lane gets the value of row nb * 32 + (lane % 32) of this wave.
+    // Fixed order of additions.  (No DMA is in flight here, so these are ordinary LDS accesses.)
+    float *red_w = red + wave * (32 * RP);
+    auto fold_lanes = [&](auto max_c, float (&tot)[NB]) {
+        constexpr bool MAXOP = decltype(max_c)::value;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) red_w[(8 * (i >> 2) + 4 * g + (i & 3)) * RP + n] = rs[nb][i];
+            __builtin_amdgcn_wave_barrier();
+            float v = MAXOP ? kNegBig : 0.f;  // each half-wave takes 16 of the row's 32 lanes' values
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const float x = red_w[n * RP + g * 16 + j];
+                v = MAXOP ? fmaxf(v, x) : v + x;
+            }
+            const float o = __shfl_xor(v, 32);
+            tot[nb] = MAXOP ? fmaxf(v, o) : (g == 0 ? v + o : o + v);  // lower half first in both halves
+            __builtin_amdgcn_wave_barrier();
+        }
+    };
+
+    // ---- common path: no max subtraction
+    sweep(std::false_type{}, std::false_type{});
+    float lt[NB], m_row[NB];
+    fold_lanes(std::false_type{}, lt);
+    bool has[NB], bad = false;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int qi = qw0 + nb * 32 + n;
+        const int thr = a.causal ? min(a.k_past + qi, a.Sk - 1) : a.Sk - 1;  // last key this row sees
+        has[nb] = (nst > 0) && (kc0 <= thr);
+        bad = bad || (has[nb] && !(lt[nb] >= 8.2718061e-25f && lt[nb] < 1.3292280e+36f));
+        m_row[nb] = has[nb] ? 0.f : kNegBig;  // an empty split must not set the merged maximum
+        if (!has[nb]) lt[nb] = 0.f;
+    }
+    {
+        const bool wbad = __builtin_amdgcn_ballot_w64(bad) != 0;
+        if (lane == 0) bad_s[wave] = wbad ? 1 : 0;
+        block_sync();
+        int any = 0;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) any |= bad_s[w];
+        bad = any != 0;  // block-uniform
+    }
+
+    // ---- rare: row maxima first, then sums with the maximum subtracted before the scale
+    if (bad) {
+        sweep(std::true_type{}, std::false_type{});
+        float mx[NB];
+        fold_lanes(std::true_type{}, mx);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            if (!has[nb]) mx[nb] = 0.f;  // no visible key in this split: every exponential is masked anyway
+            if (g == 0) mrow[wave * ROWS_W + nb * 32 + n] = mx[nb];
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) nmax[nb][i] = -mrow[wave * ROWS_W + nb * 32 + 8 * (i >> 2) + 4 * g + (i & 3)];
+        sweep(std::false_type{}, std::true_type{});
+        fold_lanes(std::false_type{}, lt);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            m_row[nb] = has[nb] ? mx[nb] : kNegBig;
+            if (!has[nb]) lt[nb] = 0.f;
+        }
+    }
+
+    // ---- store: the lower half-wave holds one row per lane
+    if (g == 0) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int qi = qw0 + nb * 32 + n;  // < rows_pad by construction
+            float2 v;
+            v.x = m_row[nb];
+            if (a.n_chunks == 1) {
+                v.y = fast_log2(lt[nb]);
+                a.lse[(int64_t)bh * a.rows_pad + qi] = v;
+            } else {
+                v.y = lt[nb];
+                a.ml[((int64_t)bh * a.n_chunks + chunk) * a.rows_pad + qi] = v;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------
 template <int D, int NB, int WAVES, bool BF>
@@ -460,6 +747,34 @@ static hipError_t launch_colstream_d(const Plan &p, const Args &a, hipStream_t s
         if (p.c_nb == 1 && p.c_waves == 4) return launch_cfg<D, 1, 4, BF>(p, a, st);
     }
     return hipErrorInvalidValue;
+}
+
+template <int D, int NB, int WAVES, bool BF>
+static hipError_t launch_rows_cfg(const Plan &p, const Args &a, hipStream_t st)
+{
+    const dim3 grid(p.n_qblk, p.n_chunks, p.B * p.H);
+    hipLaunchKernelGGL((fcs_rowstream_kernel<D, NB, WAVES, BF>), grid, dim3(64 * WAVES), 0, st, a);
+    return hipGetLastError();
+}
+
+template <int D, bool BF>
+static hipError_t launch_rowstream_d(const Plan &p, const Args &a, hipStream_t st)
+{
+    if constexpr (D <= 128) {
+        if (p.qw == 64 && p.k1_waves == 8) return launch_rows_cfg<D, 2, 8, BF>(p, a, st);
+        if (p.qw == 64 && p.k1_waves == 4) return launch_rows_cfg<D, 2, 4, BF>(p, a, st);
+    }
+    if (p.qw == 32 && p.k1_waves == 4) return launch_rows_cfg<D, 1, 4, BF>(p, a, st);
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_rowstream(const Plan &p, const Args &a, hipStream_t st)
+{
+    if (p.bf16)
+        return (p.Dp == 64) ? launch_rowstream_d<64, true>(p, a, st)
+                            : (p.Dp == 128) ? launch_rowstream_d<128, true>(p, a, st) : launch_rowstream_d<256, true>(p, a, st);
+    return (p.Dp == 64) ? launch_rowstream_d<64, false>(p, a, st)
+                        : (p.Dp == 128) ? launch_rowstream_d<128, false>(p, a, st) : launch_rowstream_d<256, false>(p, a, st);
 }
 
 hipError_t launch_colstream(const Plan &p, const Args &a, hipStream_t st)
