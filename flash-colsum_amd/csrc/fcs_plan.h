@@ -83,7 +83,8 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     // blocks fit twice.  Every further generation pays the block start (Q fragments, first key
     // stage: ~5 us) again, which nothing overlaps.
     const int target1 = (p.k1_waves == 8) ? kComputeUnits : 2 * kComputeUnits;
-    int want = (int)((target1 + base1 - 1) / base1);
+    // as many splits as still fit one generation (rounding up could start a second one for a few blocks)
+    int want = (base1 >= target1) ? 1 : (int)(target1 / base1);
     int max_chunks = ceil_div(Sk, 4 * kStageKeys);  // at least 256 keys per split
     if (want > max_chunks) want = max_chunks;
     if (want < 1) want = 1;
@@ -108,11 +109,33 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         if (groups > units) {
             // one unit per block is still too few blocks: shorter chunks (at least four stages each)
             groups = units;
-            const long want = (target + (long)B * units - 1) / ((long)B * units);
-            int c = ceil_div(ceil_div(Sk, (int)(want < 1 ? 1 : want)), kStageKeys) * kStageKeys;
+            const long want_c = target / ((long)B * units);  // rounded down: stay within one generation
+            int c = ceil_div(ceil_div(Sk, (int)(want_c < 1 ? 1 : want_c)), kStageKeys) * kStageKeys;
             if (c < 4 * kStageKeys) c = 4 * kStageKeys;
             if (c < chunk) chunk = c;
             nchunks = ceil_div(Sk, chunk);
+        } else {
+            // Blocks run in generations of `target` (what the GPU holds at once); a launch takes
+            // generations x units per block.  Among a few group counts around whole generations take
+            // the cheapest: one block over a generation would double the time of the launch.
+            const long per = (long)B * nchunks;
+            long cand[6] = {groups, target / per, 2 * target / per, 3 * target / per, 4 * target / per, units};
+            double best = 0.;
+            long best_g = groups;
+            for (int ci = 0; ci < 6; ++ci) {
+                long gcnt = cand[ci];
+                if (gcnt < 1) gcnt = 1;
+                if (gcnt > units) gcnt = units;
+                const long upg = (units + gcnt - 1) / gcnt;
+                const long g_eff = (units + upg - 1) / upg;
+                const long gens = (per * g_eff + target - 1) / target;
+                const double cost = (double)gens * ((double)upg + 0.15) + 0.0005 * (double)g_eff;
+                if (ci == 0 || cost < best) {
+                    best = cost;
+                    best_g = g_eff;
+                }
+            }
+            groups = best_g;
         }
         if (groups < 1) groups = 1;
         p.c_chunk = chunk;

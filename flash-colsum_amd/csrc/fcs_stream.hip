@@ -150,11 +150,20 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
                     const float2 *p = a.ml + bh * a.n_chunks * a.rows_pad + qi;
                     mm = kNegBig * 4.f;
                     float ll = 0.f;
-                    for (int ch = 0; ch < a.n_chunks; ++ch) {  // fixed order: bit-reproducible
-                        const float2 v = p[(int64_t)ch * a.rows_pad];
-                        const float mn = fmaxf(mm, v.x);
-                        ll = ll * fast_exp2((mm - mn) * a.c) + v.y * fast_exp2((v.x - mn) * a.c);
-                        mm = mn;
+                    for (int ch0 = 0; ch0 < a.n_chunks; ch0 += 8) {  // eight loads in flight; folded in split order
+                        float2 v[8];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            v[j].x = kNegBig * 4.f;
+                            v[j].y = 0.f;
+                            if (ch0 + j < a.n_chunks) v[j] = p[(int64_t)(ch0 + j) * a.rows_pad];
+                        }
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {  // fixed order: bit-reproducible
+                            const float mn = fmaxf(mm, v[j].x);
+                            ll = ll * fast_exp2((mm - mn) * a.c) + v[j].y * fast_exp2((v[j].x - mn) * a.c);
+                            mm = mn;
+                        }
                     }
                     lg = fast_log2(ll);
                 }
