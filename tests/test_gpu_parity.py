@@ -426,6 +426,37 @@ def test_two_streams_and_graph_replay():
         assert torch.equal(captured, want), f"replay {i}"
 
 
+def test_captured_call_owns_its_workspace():
+    """A call captured into a HIP graph must not use the per-stream workspace cache: that tensor can
+    be replaced (a larger call on the stream) or dropped (release_workspaces) while the graph still
+    replays.  Two-pass shape, so the call does use a workspace."""
+    from flash_colsum import flash_colsum_f32, _hip
+
+    q, k = _inputs((1, 4, 96, 128), (1, 4, 3000, 128), seed=31)
+    q, k = q.cuda(), k.cuda()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        eager = flash_colsum_f32(q, k, is_causal=True)  # fills the cache entry of this stream
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        captured = flash_colsum_f32(q, k, is_causal=True)
+    torch.cuda.synchronize()
+    qb, kb = _inputs((1, 8, 256, 128), (1, 8, 9000, 128), seed=32)
+    qb, kb = qb.cuda(), kb.cuda()
+    for i in range(3):
+        with torch.cuda.stream(side):
+            flash_colsum_f32(qb, kb, is_causal=True)  # grows, i.e. replaces, the cached workspace
+        _hip.release_workspaces()
+        junk = [torch.full((1 << 20,), float("nan"), device="cuda") for _ in range(8)]  # reuses whatever was freed
+        torch.cuda.synchronize()
+        captured.fill_(-1.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager), f"replay {i}"
+        del junk
+
+
 def test_explicit_k_past():
     """The causal launcher's K_past argument (reference: kernel_causal.py:94-113)."""
     from flash_colsum import _hip
