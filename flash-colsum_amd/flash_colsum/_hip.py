@@ -92,6 +92,8 @@ def _as_kernel_input(t: torch.Tensor, dtype: torch.dtype = torch.float16) -> tor
     """`dtype` (fp16 or bf16), unit last stride, 16-byte aligned rows/heads/base; copies only when it must."""
     if t.dtype != dtype:
         t = t.to(dtype)
+    if t.is_contiguous() and t.shape[-1] % 8 == 0 and t.data_ptr() % 16 == 0:
+        return t  # the common case, decided without looking at the strides one by one
     ok = (
         t.stride(3) == 1
         and t.stride(2) % 8 == 0
@@ -152,39 +154,63 @@ def release_workspaces() -> None:
         _workspaces.clear()
 
 
-def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16, general=False):
+# the raw handle of the current stream without building a torch.cuda.Stream object (absent from some builds)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _current_stream(dev: torch.device) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(dev.index)
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16, general=False, f16_only=False):
     b, h, s_q, d = q.shape
     s_k = k.shape[2]
     dev = q.device
-    out = torch.empty((b, s_k), dtype=torch.float32, device=dev)
+    n_ws = workspace_bytes(causal, b, h, s_q, s_k, d, cls_n)
+    stream = _current_stream(dev)
+    if f16_only:
+        # the caller only wants the fp16 result: the kernels' fp32 means go to the tail of the workspace
+        # instead of a tensor of their own (one allocation less per call)
+        n_head = (n_ws + 255) & ~255
+        ws = _workspace(dev, stream, n_head + 4 * b * s_k)
+        ws_ptr = ws.data_ptr()
+        out, out_ptr = None, ws_ptr + n_head
+    else:
+        out = torch.empty((b, s_k), dtype=torch.float32, device=dev)
+        ws = _workspace(dev, stream, n_ws)
+        ws_ptr, out_ptr = ws.data_ptr(), out.data_ptr()
     out_h = torch.empty((b, s_k), dtype=torch.float16, device=dev) if want_f16 else None
     out_h_ptr = out_h.data_ptr() if want_f16 else None
-    n_ws = workspace_bytes(causal, b, h, s_q, s_k, d, cls_n)
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    ws = _workspace(dev, stream, n_ws)
     qs, ks = _I64x4(*q.stride()), _I64x4(*k.stride())
     bf16 = q.dtype == torch.bfloat16
+    cdll = _lib or lib()
     if general:
-        rc = lib().fcs_colsum_general(int(bf16), int(causal), q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr,
-                                      ws.data_ptr(), n_ws, b, h, k.shape[1], s_q, s_k, d, int(cls_n), int(k_past),
-                                      qs, ks, float(scale), stream)
-        _check(rc, "fcs_colsum_general")
-        return (out, out_h) if want_f16 else out
-    if causal:
-        fn = lib().fcs_colsum_causal_bf16 if bf16 else lib().fcs_colsum_causal_f16
-        rc = fn(q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
-                h, s_q, s_k, d, int(k_past), qs, ks, float(scale), stream)
+        rc = cdll.fcs_colsum_general(int(bf16), int(causal), q.data_ptr(), k.data_ptr(), out_ptr, out_h_ptr,
+                                     ws_ptr, n_ws, b, h, k.shape[1], s_q, s_k, d, int(cls_n), int(k_past),
+                                     qs, ks, scale, stream)
+        what = "fcs_colsum_general"
+    elif causal:
+        fn = cdll.fcs_colsum_causal_bf16 if bf16 else cdll.fcs_colsum_causal_f16
+        rc = fn(q.data_ptr(), k.data_ptr(), out_ptr, out_h_ptr, ws_ptr, n_ws, h, s_q, s_k, d, int(k_past), qs, ks, scale, stream)
+        what = "fcs_colsum_causal"
     else:
-        fn = lib().fcs_colsum_noncausal_bf16 if bf16 else lib().fcs_colsum_noncausal_f16
-        rc = fn(q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h_ptr, ws.data_ptr(), n_ws,
-                b, h, s_q, d, qs, ks, float(scale), int(cls_n), stream)
-    _check(rc, ("fcs_colsum_causal" if causal else "fcs_colsum_noncausal") + ("_bf16" if bf16 else "_f16"))
+        fn = cdll.fcs_colsum_noncausal_bf16 if bf16 else cdll.fcs_colsum_noncausal_f16
+        rc = fn(q.data_ptr(), k.data_ptr(), out_ptr, out_h_ptr, ws_ptr, n_ws, b, h, s_q, d, qs, ks, scale, int(cls_n), stream)
+        what = "fcs_colsum_noncausal"
+    if rc != 0:
+        _check(rc, what if general else what + ("_bf16" if bf16 else "_f16"))
+    if f16_only:
+        return out_h
     return (out, out_h) if want_f16 else out
 
 
 def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n: int, k_past: int, want_f16: bool = False,
-            general: bool = False):
-    """Enqueue one call; returns the fp32 means, or (fp32, fp16) when `want_f16`."""
+            general: bool = False, f16_only: bool = False):
+    """Enqueue one call; returns the fp32 means, (fp32, fp16) when `want_f16`, or the fp16 tensor alone
+    when `f16_only` (which implies `want_f16`)."""
+    want_f16 = want_f16 or f16_only
     if q.device.type != "cuda" or k.device != q.device:
         raise ValueError(f"query and key must live on the same GPU, got {q.device} and {k.device}")
     # bf16 inputs run natively when both are bf16; every other dtype is converted to fp16
@@ -200,9 +226,9 @@ def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n:
     q = _as_kernel_input(q, dtype)
     k = _as_kernel_input(k, dtype)
     if q.device.index == torch.cuda.current_device():
-        return _enqueue(causal, q, k, scale, cls_n, k_past, want_f16, general)
+        return _enqueue(causal, q, k, float(scale), cls_n, k_past, want_f16, general, f16_only)
     with torch.cuda.device(q.device):
-        return _enqueue(causal, q, k, scale, cls_n, k_past, want_f16, general)
+        return _enqueue(causal, q, k, float(scale), cls_n, k_past, want_f16, general, f16_only)
 
 
 def colsum_general(Q: torch.Tensor, K: torch.Tensor, scale: float, causal: bool = False, CLS_N: int = -1,
@@ -229,7 +255,7 @@ def colsum_causal_f32(Q: torch.Tensor, K: torch.Tensor, scale: float, K_past: Op
 
 def _flash_colsum_batched(Q, K, scale, CLS_N=-1):
     """(B, S) fp16, like the reference launcher; the rounding happens in the final kernel."""
-    return _launch(False, Q, K, scale, -1 if CLS_N is None or CLS_N < 0 else int(CLS_N), 0, want_f16=True)[1]
+    return _launch(False, Q, K, scale, -1 if CLS_N is None or CLS_N < 0 else int(CLS_N), 0, f16_only=True)
 
 
 def _flash_colsum_non_batched(Q, K, scale, CLS_N=-1):
@@ -241,7 +267,7 @@ def _flash_colsum_causal(Q, K, scale, K_past=None):
     """(1, K_len) fp16; K_past defaults to max(0, K_len - Q_len)."""
     if K_past is None:
         K_past = max(0, K.shape[2] - Q.shape[2])
-    return _launch(True, Q, K, scale, -1, int(K_past), want_f16=True)[1]
+    return _launch(True, Q, K, scale, -1, int(K_past), f16_only=True)
 
 
 TOPK_SORT_MAX = 4096  # FCS_TOPK_SORT_MAX of include/flash_colsum.h
@@ -258,7 +284,7 @@ def topk_f32(means: torch.Tensor, k: int, sorted: bool = True):
     val = torch.empty((b, k), dtype=torch.float32, device=means.device)
     in_kernel_sort = sorted and k <= TOPK_SORT_MAX
     with torch.cuda.device(means.device):
-        stream = torch.cuda.current_stream(means.device).cuda_stream
+        stream = _current_stream(means.device)
         _check(lib().fcs_topk_f32(means.data_ptr(), b, s, int(k), idx.data_ptr(), val.data_ptr(), int(in_kernel_sort), stream),
                "fcs_topk_f32")
     if sorted and not in_kernel_sort:
@@ -278,7 +304,7 @@ def threshold_f32(means: torch.Tensor, tau: float):
     idx = torch.empty((b, s), dtype=torch.int64, device=means.device)
     cnt = torch.empty((b,), dtype=torch.int32, device=means.device)
     with torch.cuda.device(means.device):
-        stream = torch.cuda.current_stream(means.device).cuda_stream
+        stream = _current_stream(means.device)
         _check(lib().fcs_threshold_f32(means.data_ptr(), b, s, float(tau), idx.data_ptr(), cnt.data_ptr(), stream),
                "fcs_threshold_f32")
     return idx, cnt
