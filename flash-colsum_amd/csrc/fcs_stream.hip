@@ -70,11 +70,31 @@ __device__ __forceinline__ int row_swizzle(int row)
 // source of the 16-byte pieces that lie past the tensor's head dim (kernels compiled for a wider head)
 __device__ unsigned int g_zero_piece[4];
 
+// ceiling of a row's sum of exponentials in the pre-scaled variants: keeps every score of the common path
+// below 28 in the exponent's unit, which bounds what rounding Q * c to fp16 can do to it
+constexpr float kRowSumHiPre = 268435456.f;  // 2^28
+
+// Pre-scaled stationary operand: q * cs in fp32, rounded to fp16 (cs = c with the scale's sign).  The
+// scores then leave the matrix pipe in the exponent's unit and the per-score multiply disappears.  Both
+// passes form the operand with this one function, so they see the same score bits.
+__device__ __forceinline__ half8 prescale(half8 v, float cs)
+{
+    half8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (_Float16)((float)v[e] * cs);
+    return r;
+}
+
 }  // namespace
 
-template <int D, int NB, int WAVES, bool BF>
+// PRE (fp16, D = 64 only; chosen by the launcher when at least 4096 (head, row) pairs are averaged and
+// |scale| <= 1/8): the stationary operand is Q * c rounded to fp16, the row constant is -log2 l_i, and
+// p_ij = 2^(s'_ij - log2 l_i) costs a v_exp_f32 alone.  Pass 1 made l_i from the same pre-scaled scores.
+// Units with a stabilised row keep the raw operand and the two-constant form.
+template <int D, int NB, int WAVES, bool BF, bool PRE>
 __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args a)
 {
+    static_assert(!PRE || (!BF && D == 64), "the pre-scaled variant exists for fp16 operands and 64-wide heads");
     constexpr int THREADS = 64 * WAVES;
     constexpr int NT = D / 16;                 // MFMA steps along the head dim
     constexpr int KT = kStageKeys;             // 64 keys per stage
@@ -167,7 +187,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
                     }
                     lg = fast_log2(ll);
                 }
-                nl = (a.c == 0.f) ? -lg : -lg / a.c;
+                nl = (PRE || a.c == 0.f) ? -lg : -lg / a.c;
             }
             // a stabilised row anywhere in the unit switches the whole unit to the two-constant form
             const bool sh = __builtin_amdgcn_ballot_w64(mm != 0.f) != 0;
@@ -191,7 +211,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
                 for (int t = 0; t < NT; ++t) {
                     half8 v = kZero8;  // channels past the tensor's head dim are zeros
                     if (t * 16 + g * 8 < a.D) v = load8(row + t * 16);
-                    if (a.negate) v = flip_sign(v);
+                    if (!PRE && a.negate) v = flip_sign(v);
                     if (a.c == 0.f) v = kZero8;
                     qf[nb][t] = v;
                 }
@@ -263,6 +283,15 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
             asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(f) : "v"(ad) : "memory");
             shifted = __builtin_amdgcn_ballot_w64(f != 0) != 0;
         }
+        if (PRE) {  // block-uniform choice: scaled operand, or the raw one (with the scale's sign) for the two-constant form
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    if (!shifted) qf[nb][t] = prescale(qf[nb][t], a.negate ? -a.c : a.c);
+                    else if (a.negate) qf[nb][t] = flip_sign(qf[nb][t]);
+                }
+        }
         floatx16 cinit[NB];  // row constants in accumulator layout: register i <-> row 8*(i/4) + 4*g + i%4
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
@@ -331,7 +360,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
             } else {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const float pr = fast_exp2(sc[i] * cmul);
+                    const float pr = fast_exp2(PRE ? sc[i] : sc[i] * cmul);
                     cp[i & 3] += (rel <= nb * 32 + 8 * (i >> 2) + (i & 3)) ? pr : 0.f;
                 }
             }
@@ -365,7 +394,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
         };
         auto drain_fast = [&](const floatx16 &sc) {  // every key of the tile visible, no stabilised row
 #pragma unroll
-            for (int i = 0; i < 16; ++i) cp[i & 3] += fast_exp2(sc[i] * cmul);
+            for (int i = 0; i < 16; ++i) cp[i & 3] += fast_exp2(PRE ? sc[i] : sc[i] * cmul);
         };
 
         // one stage, in ring slot SLOT (compile-time)
@@ -456,9 +485,12 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
 // [2^-80, 2^120); a block that leaves that range redoes its keys in two more sweeps (row maxima, then
 // sums of 2^((s - m) * c), the maximum subtracted before the scale).  Writes (m, log2 l) per row, or
 // (m, l) per (split, row) when the keys are split; the column pass merges the splits.
-template <int D, int NB, int WAVES, bool BF>
+// PRE: see the column pass.  The common sweep runs on Q * c rounded to fp16 and accepts row sums below
+// 2^28 only; a block that leaves the range reloads the raw operand for its stabilised sweeps.
+template <int D, int NB, int WAVES, bool BF, bool PRE>
 __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args a)
 {
+    static_assert(!PRE || (!BF && D == 64), "the pre-scaled variant exists for fp16 operands and 64-wide heads");
     constexpr int THREADS = 64 * WAVES;
     constexpr int NT = D / 16;
     constexpr int KT = kStageKeys;
@@ -506,19 +538,24 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
         take[t] = lds_addr(ring) + (uint32_t)(n * ROW_BYTES + (((2 * t + g) ^ row_swizzle<D>(n)) * 16));
 
     half8 qf[NB][NT];
-    {
+    auto load_q = [&](bool scaled) {  // this wave's query rows: pre-scaled, or raw with the scale's sign
         const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
+        int lane_o = lane;
+        asm volatile("" : "+v"(lane_o));  // addresses are formed here, not kept for a second call
+        const int n_o = lane_o & 31, g_o = lane_o >> 5;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-            const _Float16 *row = qp + (int64_t)min(qw0 + nb * 32 + n, a.Sq - 1) * a.qs_s + g * 8;
+            const _Float16 *row = qp + (int64_t)min(qw0 + nb * 32 + n_o, a.Sq - 1) * a.qs_s + g_o * 8;
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 half8 v = kZero8;
-                if (t * 16 + g * 8 < a.D) v = load8(row + t * 16);
-                qf[nb][t] = a.negate ? flip_sign(v) : v;
+                if (t * 16 + g_o * 8 < a.D) v = load8(row + t * 16);
+                if (PRE && scaled) qf[nb][t] = prescale(v, a.negate ? -a.c : a.c);
+                else qf[nb][t] = a.negate ? flip_sign(v) : v;
             }
         }
-    }
+    };
+    load_q(true);
     const char *kp = reinterpret_cast<const char *>(a.k + (int64_t)b * a.ks_b +
                                                     (int64_t)kv_head(h, a.kv_group, a.kv_magic) * a.ks_h);
     const int64_t k_row_b = a.ks_s * 2;
@@ -572,6 +609,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
     auto sweep = [&](auto max_c, auto shift_c) {
         constexpr bool MAXOP = decltype(max_c)::value;
         constexpr bool SHIFT = decltype(shift_c)::value;
+        constexpr bool SCALED = PRE && !MAXOP && !SHIFT;  // the common sweep of the pre-scaled variant
         constexpr int TILES = NA * NB;
         static_assert(NA == 2 && TILES % 2 == 0, "fragment offsets and the two alternating accumulators");
 #pragma unroll
@@ -593,7 +631,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     if (MAXOP) rs[nb][i] = fmaxf(rs[nb][i], sc[i]);
-                    else rs[nb][i] += fast_exp2((SHIFT ? sc[i] + nmax[nb][i] : sc[i]) * cmul);
+                    else rs[nb][i] += SCALED ? fast_exp2(sc[i]) : fast_exp2((SHIFT ? sc[i] + nmax[nb][i] : sc[i]) * cmul);
                 }
             } else {
                 const int key = kb_t + na * 32 + n;
@@ -603,7 +641,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
                 for (int i = 0; i < 16; ++i) {
                     const bool vis = rel <= nb * 32 + 8 * (i >> 2) + (i & 3);
                     if (MAXOP) rs[nb][i] = fmaxf(rs[nb][i], vis ? sc[i] : kNegBig);
-                    else rs[nb][i] += vis ? fast_exp2((SHIFT ? sc[i] + nmax[nb][i] : sc[i]) * cmul) : 0.f;
+                    else rs[nb][i] += vis ? (SCALED ? fast_exp2(sc[i]) : fast_exp2((SHIFT ? sc[i] + nmax[nb][i] : sc[i]) * cmul)) : 0.f;
                 }
             }
         };
@@ -677,7 +715,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
         const int qi = qw0 + nb * 32 + n;
         const int thr = a.causal ? min(a.k_past + qi, a.Sk - 1) : a.Sk - 1;  // last key this row sees
         has[nb] = (nst > 0) && (kc0 <= thr);
-        bad = bad || (has[nb] && !(lt[nb] >= 8.2718061e-25f && lt[nb] < 1.3292280e+36f));
+        bad = bad || (has[nb] && !(lt[nb] >= 8.2718061e-25f && lt[nb] < (PRE ? kRowSumHiPre : 1.3292280e+36f)));
         m_row[nb] = has[nb] ? 0.f : kNegBig;  // an empty split must not set the merged maximum
         if (!has[nb]) lt[nb] = 0.f;
     }
@@ -693,6 +731,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
 
     // ---- rare: row maxima first, then sums with the maximum subtracted before the scale
     if (bad) {
+        if (PRE) load_q(false);
         sweep(std::true_type{}, std::false_type{});
         float mx[NB];
         fold_lanes(std::true_type{}, mx);
@@ -736,11 +775,25 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
 // ------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------
+// Both passes must agree on the pre-scaled variant: fp16 operands, 64-wide kernels, |scale| <= 1/8, and
+// at least 4096 (head, row) pairs averaged per output (the rounding of Q * c to fp16 perturbs every
+// score by about 2^-12 relative; over that many rows its effect on a mean stays below 1e-4 relative).
+static bool stream_prescaled(const Plan &p, const Args &a)
+{
+    return !p.bf16 && p.Dp == 64 && a.c != 0.f && fabsf(a.c) <= 0.1251f * 1.44269504f && (long)p.H * p.q_rows >= 4096;
+}
+
 template <int D, int NB, int WAVES, bool BF>
 static hipError_t launch_cfg(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.c_nchunks, p.c_groups, p.B);
-    hipLaunchKernelGGL((fcs_colstream_kernel<D, NB, WAVES, BF>), grid, dim3(64 * WAVES), 0, st, a);
+    if constexpr (D == 64 && !BF) {
+        if (stream_prescaled(p, a)) {
+            hipLaunchKernelGGL((fcs_colstream_kernel<D, NB, WAVES, BF, true>), grid, dim3(64 * WAVES), 0, st, a);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((fcs_colstream_kernel<D, NB, WAVES, BF, false>), grid, dim3(64 * WAVES), 0, st, a);
     return hipGetLastError();
 }
 
@@ -762,7 +815,13 @@ template <int D, int NB, int WAVES, bool BF>
 static hipError_t launch_rows_cfg(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.n_qblk, p.n_chunks, p.B * p.H);
-    hipLaunchKernelGGL((fcs_rowstream_kernel<D, NB, WAVES, BF>), grid, dim3(64 * WAVES), 0, st, a);
+    if constexpr (D == 64 && !BF) {
+        if (stream_prescaled(p, a)) {
+            hipLaunchKernelGGL((fcs_rowstream_kernel<D, NB, WAVES, BF, true>), grid, dim3(64 * WAVES), 0, st, a);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((fcs_rowstream_kernel<D, NB, WAVES, BF, false>), grid, dim3(64 * WAVES), 0, st, a);
     return hipGetLastError();
 }
 

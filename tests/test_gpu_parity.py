@@ -274,6 +274,30 @@ def test_prescaled_shared_q_variant(shape, same, kw, boost):
     _assert_close(_run(q, k, **kw), _oracle(q, k, **kw), f"prescaled {shape} same={same} {kw} boost={boost}")
 
 
+@pytest.mark.parametrize("qs,ks,kw,same,boost", [
+    ((1, 4, 4096, 64), (1, 4, 4096, 64), {}, False, 0.0),                        # non-causal, keys split in pass 1
+    ((1, 4, 4096, 64), (1, 4, 4096, 64), {"scale": -0.125}, False, 0.0),         # the sign rides on the operand
+    ((2, 8, 2100, 64), (2, 8, 2100, 64), {}, False, 0.0),                        # ragged, just past the fused kernel's range
+    ((1, 16, 700, 64), (1, 16, 5000, 64), {"is_causal": True}, False, 0.0),      # causal, D = 64
+    ((1, 8, 600, 48), (1, 8, 3000, 48), {"is_causal": True}, False, 0.0),        # narrower head in the 64-wide kernels
+    ((1, 4, 4096, 64), (1, 4, 4096, 64), {}, False, 6.0),                        # some rows leave the 2^28 range: raw-operand sweeps
+    ((1, 4, 4096, 64), (1, 4, 4096, 64), {}, True, 40.0),                        # ... far out, Q == K
+    ((1, 32, 200, 64), (1, 32, 9000, 64), {"is_causal": True}, False, 8.0),      # ... with split keys and the causal edge
+    ((1, 4, 4096, 64), (1, 4, 4096, 64), {"scale": 0.2}, False, 0.0),            # scale above 1/8: the exact variant
+    ((1, 2, 1000, 64), (1, 2, 4000, 64), {"is_causal": True}, False, 0.0),       # fewer than 4096 pairs: the exact variant
+])
+def test_prescaled_streaming_variant(qs, ks, kw, same, boost):
+    """Two-pass calls with fp16 operands, 64-wide kernels, |scale| <= 1/8 and >= 4096 averaged (head, row)
+    pairs run both passes on Q * c rounded to fp16; blocks whose row sums reach 2^28 (or fall below
+    2^-80) must redo their keys on the raw operand, and the column pass must follow them there."""
+    q, k = _inputs(qs, ks, seed=13, same=same)
+    if boost:
+        q[:, 1, 100:164] *= boost
+        if same:
+            k = q.clone()
+    _assert_close(_run(q, k, **kw), _oracle(q, k, **kw), f"prescaled streaming {qs} {ks} {kw} same={same} boost={boost}")
+
+
 @pytest.mark.parametrize("qs,ks,kw", [
     ((4, 8, 512, 64), (4, 8, 512, 64), {}),                          # fused, whole tiles
     ((8, 2, 2048, 64), (8, 2, 2048, 64), {}),                        # fused, where fp16 would take the pre-scaled variant
