@@ -278,17 +278,19 @@ def test_prescaled_shared_q_variant(shape, same, kw, boost):
     ((1, 4, 4096, 64), (1, 4, 4096, 64), {}, False, 0.0),                        # non-causal, keys split in pass 1
     ((1, 4, 4096, 64), (1, 4, 4096, 64), {"scale": -0.125}, False, 0.0),         # the sign rides on the operand
     ((2, 8, 2100, 64), (2, 8, 2100, 64), {}, False, 0.0),                        # ragged, just past the fused kernel's range
-    ((1, 16, 700, 64), (1, 16, 5000, 64), {"is_causal": True}, False, 0.0),      # causal, D = 64
-    ((1, 8, 600, 48), (1, 8, 3000, 48), {"is_causal": True}, False, 0.0),        # narrower head in the 64-wide kernels
-    ((1, 4, 4096, 64), (1, 4, 4096, 64), {}, False, 6.0),                        # some rows leave the 2^28 range: raw-operand sweeps
+    ((1, 16, 700, 64), (1, 16, 5000, 64), {"is_causal": True}, False, 0.0),      # causal: always the exact variant
+    ((2, 8, 2500, 48), (2, 8, 2500, 48), {}, False, 0.0),                        # narrower head in the 64-wide kernels
+    ((1, 8, 3000, 64), (1, 8, 3000, 64), {"cls_len": 2500}, False, 0.0),         # 20000 averaged pairs
+    ((1, 4, 3000, 64), (1, 4, 3000, 64), {"cls_len": 1500}, False, 0.0),         # 6000 averaged pairs: the exact variant
+    ((1, 4, 4096, 64), (1, 4, 4096, 64), {}, False, 6.0),                        # some rows leave the 2^20 range: raw-operand sweeps
     ((1, 4, 4096, 64), (1, 4, 4096, 64), {}, True, 40.0),                        # ... far out, Q == K
-    ((1, 32, 200, 64), (1, 32, 9000, 64), {"is_causal": True}, False, 8.0),      # ... with split keys and the causal edge
+    ((3, 8, 2304, 64), (3, 8, 2304, 64), {}, False, 8.0),                        # ... batched
     ((1, 4, 4096, 64), (1, 4, 4096, 64), {"scale": 0.2}, False, 0.0),            # scale above 1/8: the exact variant
-    ((1, 2, 1000, 64), (1, 2, 4000, 64), {"is_causal": True}, False, 0.0),       # fewer than 4096 pairs: the exact variant
+    ((1, 2, 4096, 64), (1, 2, 4096, 64), {}, False, 0.0),                        # fewer than 16384 pairs: the exact variant
 ])
 def test_prescaled_streaming_variant(qs, ks, kw, same, boost):
-    """Two-pass calls with fp16 operands, 64-wide kernels, |scale| <= 1/8 and >= 4096 averaged (head, row)
-    pairs run both passes on Q * c rounded to fp16; blocks whose row sums reach 2^28 (or fall below
+    """Non-causal two-pass calls with fp16 operands, 64-wide kernels, |scale| <= 1/8 and >= 16384 averaged
+    (head, row) pairs run both passes on Q * c rounded to fp16; blocks whose row sums reach 2^20 (or fall below
     2^-80) must redo their keys on the raw operand, and the column pass must follow them there."""
     q, k = _inputs(qs, ks, seed=13, same=same)
     if boost:
@@ -296,6 +298,18 @@ def test_prescaled_streaming_variant(qs, ks, kw, same, boost):
         if same:
             k = q.clone()
     _assert_close(_run(q, k, **kw), _oracle(q, k, **kw), f"prescaled streaming {qs} {ks} {kw} same={same} boost={boost}")
+
+
+@pytest.mark.parametrize("amp", [1.0, 1.6, 2.0, 2.5])
+def test_prescaled_variants_against_input_amplitude(amp):
+    """The error of a pre-scaled score grows with the spread of the scores; the row-sum ceilings (2^20 in
+    the streaming kernels, 2^28 in the fused one) must send peaked rows to the exact sweeps before the
+    means leave the bar.  Few heads, so that a column is not averaged over many rows."""
+    for shape in [(1, 4, 4096, 64), (2, 4, 1024, 64)]:
+        g = torch.Generator().manual_seed(5)
+        q = (torch.randn(shape, generator=g) * amp).half()
+        k = (torch.randn(shape, generator=g) * amp).half()
+        _assert_close(_run(q, k, scale=0.125), _oracle(q, k, scale=0.125), f"amplitude {amp} {shape}")
 
 
 @pytest.mark.parametrize("qs,ks,kw", [
