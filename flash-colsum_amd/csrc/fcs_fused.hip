@@ -361,7 +361,10 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // PRE: the Q item of a head is not a tile in the ring but this wave's 32 / PRE rows of its query
     // group's raw tile (512 B or 1 KB), one ordinary 8- or 16-byte load per lane; the wave scales
     // them and publishes them in `qshare`.
-    uint4v qraw = {0u, 0u, 0u, 0u};
+    // raw Q rows of the pre-scaled variant: written by an asynchronous load and read after a hand-placed
+    // wait, so the variable the load names must be the one the wait names (no copies in between)
+    typedef uint32_t qraw_t __attribute__((ext_vector_type(PRE == 8 ? 2 : 4)));
+    qraw_t qraw = {};
     auto item_vm = [&](int j_ahead) { return (PRE && (j_ahead % ITEMS) == 0) ? 1 : NT; };  // VMEM instructions of an item
     // byte offsets of the key heads of the current and of the next query head (grouped key heads:
     // head / kv_group), refreshed once per head instead of at every fetch
@@ -389,13 +392,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 } else {
                     src = q_b + (int64_t)hh * q_head_b + ((PRE == 8) ? kg * 512 + lane * 8 : kg * 1024 + lane * 16);
                 }
-                if (PRE == 8) {
-                    const uint2 v = *reinterpret_cast<const uint2 *>(src);
-                    qraw[0] = v.x;
-                    qraw[1] = v.y;
-                } else {
-                    qraw = *reinterpret_cast<const uint4v *>(src);
-                }
+                // Issued from inline assembly, so that the compiler does not count it among the loads
+                // it waits for itself: it cannot tell how many DMA fetches were issued behind this
+                // load and would drain all of them (vmcnt(0)) before the first use.  q_publish waits
+                // for exactly this load.
+                if (PRE == 8) asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(qraw) : "v"(src) : "memory");
+                else asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qraw) : "v"(src) : "memory");
             }
         } else if (j == 0)
             fetch_piece(true, q_b + (int64_t)hh * q_head_b, q_row_b, q_voff, 0, 0, slot, tt);
@@ -441,9 +443,13 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // their swizzled place in the query group's tile of qshare[buf]; a workgroup barrier must
     // follow before they are read
     auto q_publish = [&](int buf) {
+        // the raw rows were requested one item before the two most recent fetches (2 * NT DMA
+        // instructions): once at most those are outstanding, the rows have landed
+        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(qraw) : "n"(2 * NT) : "memory");
         const float cs = a.negate ? -a.c : a.c;
-        const half8 raw = __builtin_bit_cast(half8, qraw);
-        half8 sc;
+        typedef _Float16 qhalf_t __attribute__((ext_vector_type(PRE == 8 ? 4 : 8)));
+        const qhalf_t raw = __builtin_bit_cast(qhalf_t, qraw);
+        half8 sc = kZero8;
 #pragma unroll
         for (int e = 0; e < (PRE == 8 ? 4 : 8); ++e) sc[e] = (_Float16)((float)raw[e] * cs);
         char *tile = qshare + (buf * PQG + qg) * 4096;
