@@ -93,6 +93,7 @@ int run(int bf16, int causal, const void *q, const void *k, float *out, void *ou
     a.inv_norm = 1.0f / ((float)H * (float)p.q_rows);
     a.n_partials = p.n_partials;
     a.f_kg = p.f_kg; a.f_tpw = p.f_tpw; a.f_nqblk = p.f_nqblk; a.f_hpg = p.f_hpg;
+    a.f_rbpw = p.f_rbpw; a.f_nwgq = p.f_nwgq;
     return fcs::launch_colsum(p, a, stream);
 }
 

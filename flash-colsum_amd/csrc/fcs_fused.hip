@@ -237,20 +237,22 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     const int qg = wave / kg_n, kg = wave - qg * kg_n;
     // The row blocks of one (head group, batch entry) read the same K: they run on one XCD, close
     // together in time.
-    int hgi, b, qblk;
+    int hgi, b, qwg;
     {
         int bx, by, bz;
         xcd_contiguous_block(bx, by, bz);
-        qblk = bx % a.f_nqblk;
-        b = bx / a.f_nqblk;
+        qwg = bx % a.f_nwgq;
+        b = bx / a.f_nwgq;
         hgi = by;
     }
+    // A workgroup walks over units = (head, row block): the heads of its head group, and for each of
+    // them its f_rbpw adjacent row blocks (row blocks innermost: the head's keys are fetched into the
+    // L2 once and re-read from there; the workgroups of an XCD walk in step, so they read the same
+    // head's keys at the same time).  Every unit adds into the same column sums.
     const int h_begin = hgi * a.f_hpg, h_end = min(a.H, h_begin + a.f_hpg);
-    const int n_units = h_end - h_begin;
-    const int blk_row0 = qblk * 32 * qg_n;  // first query row of the block
-    // first query row of this wave; a wave whose rows all lie past the tensor re-reads the last row
-    // (its rows carry weight 0)
-    const int q0 = min(blk_row0 + qg * 32, a.Sq - 1);
+    const int n_heads = h_end - h_begin;
+    const int rb_first = qwg * a.f_rbpw, rb_n = min(a.f_rbpw, a.f_nqblk - rb_first);
+    const int n_units = rb_n * n_heads;
     const int kbase = kg * TPW * 32;        // first key of this wave
 
     RowRed rr;
@@ -280,8 +282,6 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // a wave's rows (and whole tiles of them) may lie past the end of the tensor.
     const char *q_batch = reinterpret_cast<const char *>(a.q + (int64_t)b * a.qs_b);
     const char *k_batch = reinterpret_cast<const char *>(a.k + (int64_t)b * a.ks_b);
-    const int q_first = blk_row0 + qg * 32;  // this wave's first query row, unclamped
-    const char *q_b = q_batch + (int64_t)q0 * q_row_b;
     const char *k_b = k_batch + (int64_t)min(kbase, a.Sk - 1) * k_row_b;
     const int64_t q_head_b = a.qs_h * 2, k_head_b = a.ks_h * 2;
     char *my_ring = ring + wave * (NS * SLOT_BYTES);
@@ -366,19 +366,39 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     typedef uint32_t qraw_t __attribute__((ext_vector_type(PRE == 8 ? 2 : 4)));
     qraw_t qraw = {};
     auto item_vm = [&](int j_ahead) { return (PRE && (j_ahead % ITEMS) == 0) ? 1 : NT; };  // VMEM instructions of an item
-    // byte offsets of the key heads of the current and of the next query head (grouped key heads:
-    // head / kv_group), refreshed once per head instead of at every fetch
-    constexpr int HEADS_AHEAD = (ITEMS + NS - 1) / ITEMS;  // the look-ahead reaches this many heads past the current one
+    // What the fetches need to know of the current unit and of the units the look-ahead reaches,
+    // refreshed once per unit instead of at every fetch: the head's Q slice, the wave's first query
+    // row (unclamped; a wave whose rows all lie past the tensor re-reads the last row, its rows carry
+    // weight 0), the wave's Q tile, and the byte offset of the key head (grouped key heads: head /
+    // kv_group).  Past the last unit the entries repeat it.
+    constexpr int HEADS_AHEAD = (ITEMS + NS - 1) / ITEMS;  // the look-ahead reaches this many units past the current one
+    const char *u_qhead[HEADS_AHEAD + 1];
+    const char *u_qtile[HEADS_AHEAD + 1];
+    int u_qfirst[HEADS_AHEAD + 1];
     int64_t k_off[HEADS_AHEAD + 1];
-    auto set_k_off = [&](int h_now) {
+    int cur_rb = 0, cur_hr = 0;  // row block (relative) and head (relative) of the current unit
+    auto set_units = [&]() {
+        int r = cur_rb, hr = cur_hr;
 #pragma unroll
-        for (int i = 0; i <= HEADS_AHEAD; ++i)
-            k_off[i] = (int64_t)kv_head(min(h_now + i, h_end - 1), a.kv_group, a.kv_magic) * k_head_b;
+        for (int i = 0; i <= HEADS_AHEAD; ++i) {
+            const int hh = h_begin + hr;
+            const int first = ((rb_first + r) * qg_n + qg) * 32;
+            u_qfirst[i] = first;
+            u_qhead[i] = q_batch + (int64_t)hh * q_head_b;
+            u_qtile[i] = u_qhead[i] + (int64_t)min(first, a.Sq - 1) * q_row_b;
+            k_off[i] = (int64_t)kv_head(hh, a.kv_group, a.kv_magic) * k_head_b;
+            if (r != rb_n - 1 || hr != n_heads - 1) {
+                if (++r == rb_n) {
+                    r = 0;
+                    ++hr;
+                }
+            }
+        }
     };
-    set_k_off(h_begin);
-    auto fetch_pos_piece = [&](int h_now, int j_ahead /* item index counted from the Q tile of head h_now, compile-time */,
+    set_units();
+    auto fetch_pos_piece = [&](int j_ahead /* item index counted from the Q tile of the current unit, compile-time */,
                                int slot, int tt) {
-        const int hh = min(h_now + j_ahead / ITEMS, h_end - 1);
+        const int ua = j_ahead / ITEMS;
         const int j = j_ahead % ITEMS;
         if (j == 0 && PRE) {
             if (tt == 0) {
@@ -388,9 +408,9 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 if (RAGGED) {
                     const int row_in_tile = (PRE == 8) ? kg * 4 + (lane >> 4) : kg * 8 + (lane >> 3);
                     const int in_row_b = (PRE == 8) ? (lane & 15) * 8 : (lane & 7) * 16;
-                    src = q_batch + (int64_t)hh * q_head_b + (size_t)min(q_first + row_in_tile, a.Sq - 1) * q_row_b + in_row_b;
+                    src = u_qhead[ua] + (size_t)min(u_qfirst[ua] + row_in_tile, a.Sq - 1) * q_row_b + in_row_b;
                 } else {
-                    src = q_b + (int64_t)hh * q_head_b + ((PRE == 8) ? kg * 512 + lane * 8 : kg * 1024 + lane * 16);
+                    src = u_qtile[ua] + ((PRE == 8) ? kg * 512 + lane * 8 : kg * 1024 + lane * 16);
                 }
                 // Issued from inline assembly, so that the compiler does not count it among the loads
                 // it waits for itself: it cannot tell how many DMA fetches were issued behind this
@@ -400,24 +420,24 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 else asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qraw) : "v"(src) : "memory");
             }
         } else if (j == 0)
-            fetch_piece(true, q_b + (int64_t)hh * q_head_b, q_row_b, q_voff, 0, 0, slot, tt);
+            fetch_piece(true, u_qtile[ua], q_row_b, q_voff, 0, 0, slot, tt);
         else
-            fetch_piece(true, k_b + k_off[j_ahead / ITEMS] + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff, 0, 0, slot, tt);
+            fetch_piece(true, k_b + k_off[ua] + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff, 0, 0, slot, tt);
     };
-    auto fetch_pos = [&](int h_now, int j_ahead, int slot) {
+    auto fetch_pos = [&](int j_ahead, int slot) {
         if (RAGGED) {
             // One wave-uniform decision per tile: a tile that lies wholly inside its tensor and has
             // dense rows takes the cheap whole-tile form; only tiles that touch the end (or strided
             // rows) pay for per-lane row clamping.
-            const int hh = min(h_now + j_ahead / ITEMS, h_end - 1);
+            const int ua = j_ahead / ITEMS;
             const int j = j_ahead % ITEMS;
             const bool is_q = (j == 0);
             if (PRE && is_q) {  // the Q item of the pre-scaled variant is a plain load, not a tile
-                fetch_pos_piece(h_now, j_ahead, slot, 0);
+                fetch_pos_piece(j_ahead, slot, 0);
                 return;
             }
-            const char *slice = is_q ? q_batch + (int64_t)hh * q_head_b : k_batch + k_off[j_ahead / ITEMS];
-            const int first_row = is_q ? q_first : kbase + (j - 1) * 32, n_rows = is_q ? a.Sq : a.Sk;
+            const char *slice = is_q ? u_qhead[ua] : k_batch + k_off[ua];
+            const int first_row = is_q ? u_qfirst[ua] : kbase + (j - 1) * 32, n_rows = is_q ? a.Sq : a.Sk;
             const uint32_t row_b = is_q ? q_row_b : k_row_b;
             if (first_row + 32 <= n_rows && row_b == (uint32_t)(D * 2)) {
                 const char *tile = slice + (size_t)first_row * (D * 2);
@@ -429,7 +449,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             }
         } else {
 #pragma unroll
-            for (int tt = 0; tt < NT; ++tt) fetch_pos_piece(h_now, j_ahead, slot, tt);
+            for (int tt = 0; tt < NT; ++tt) fetch_pos_piece(j_ahead, slot, tt);
         }
     };
     int sq = 0;  // ring slot of the current head's Q tile (only used when the slots are not static)
@@ -474,15 +494,17 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 
     half8 qf[NT], kf[2][NT];
 #pragma unroll
-    for (int i = 0; i < NS; ++i) fetch_pos(h_begin, i, i);
+    for (int i = 0; i < NS; ++i) fetch_pos(i, i);
     if (PRE) {
         q_publish(0);
         __syncthreads();
     }
 
     for (int unit = 0; unit < n_units; ++unit) {
-        const int h = h_begin + unit;
-        set_k_off(h);
+        const int h = h_begin + cur_hr;
+        const int blk_row0 = (rb_first + cur_rb) * 32 * qg_n;  // first query row of the unit's row block
+        const int q_first = blk_row0 + qg * 32;                  // this wave's first query row, unclamped
+        set_units();
         // this head's Q tile and first key tile (fetched during the previous head).  (Reading them
         // back earlier, under the previous head's column-sum FMAs, makes them live across the loop
         // and the kernel spills.)
@@ -545,11 +567,11 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 #pragma unroll
                     for (int tt = 0; tt < NT; ++tt) qf[tt] = flip_sign(qf[tt]);
                 }
-                fetch_pos(h, 0 + NS, slot_of(0));
-                fetch_pos(h, 1 + NS, slot_of(1));
+                fetch_pos(0 + NS, slot_of(0));
+                fetch_pos(1 + NS, slot_of(1));
             } else {
                 take_wait(kf[t & 1]);
-                fetch_pos(h, 1 + t + NS, slot_of(1 + t));
+                fetch_pos(1 + t + NS, slot_of(1 + t));
             }
             // the next key tile has landed; the two items fetched after it may be in flight
             if (item_vm(t + 3) + item_vm(t + 4) == 2 * NT) FCS_WAIT_VM(2 * NT);
@@ -661,11 +683,15 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                     if (u == t) col_acc[u] += sum;
             }
         }
+        if (++cur_rb == rb_n) {
+            cur_rb = 0;
+            ++cur_hr;
+        }
     }
     FCS_WAIT_VM(0);  // drain the look-ahead fetches before the block's LDS is released
 
     // ---------------- the two half-waves hold different rows of the same keys: add, then store
-    const int slab = (hgi * a.f_nqblk + qblk) * qg_n + qg;
+    const int slab = (hgi * a.f_nwgq + qwg) * qg_n + qg;
     float *dst = a.partial + ((int64_t)slab * a.B + b) * a.Sk;
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
@@ -678,7 +704,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 template <int TPW, bool BF>
 static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
-    const dim3 grid(p.f_nqblk * p.B, p.f_hg);  // x = batch entry * f_nqblk + row block
+    const dim3 grid(p.f_nwgq * p.B, p.f_hg);  // x = batch entry * f_nwgq + workgroup along the query axis
     const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
     const bool pre = !BF && TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4) && (long)p.H * p.q_rows >= 4096 &&
                      fabsf(a.c) <= 0.1251f * 1.44269504f;

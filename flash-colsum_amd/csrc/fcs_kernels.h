@@ -37,6 +37,8 @@ struct Args {
     int f_tpw;       // 32-key tiles per wave (<= 8)
     int f_nqblk;     // blocks along the query axis (32 * 8 / f_kg rows each)
     int f_hpg;       // heads per block
+    int f_rbpw;      // adjacent row blocks per block (a block walks over f_rbpw x f_hpg units)
+    int f_nwgq;      // blocks along the query axis: ceil(f_nqblk / f_rbpw)
 };
 
 // Enqueues every kernel of one call on `stream`; returns 0 or the hipError_t of a failed launch.

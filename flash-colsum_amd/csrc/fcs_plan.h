@@ -42,13 +42,15 @@ struct Plan {
     int c_chunk, c_nchunks;
     int c_groups, c_upg;
     // fused single-kernel path: non-causal, all keys of a row block fit in one
-    // workgroup's registers.  grid = (f_nqblk * B, f_hg)
+    // workgroup's registers.  grid = (f_nwgq * B, f_hg)
     int fewrows;     // 1: few-rows path (non-causal, q_rows <= 4): grid = B * f_hg, slabs = f_hg
     int fused;       // 1: use it (then the two-pass fields above are unused)
     int f_kg, f_qg;  // waves along keys / along queries, f_kg * f_qg == 8
     int f_tpw;       // 32-key tiles per wave
     int f_nqblk;     // query blocks of 32 * f_qg rows
     int f_hg, f_hpg; // head groups, heads per group
+    int f_rbpw;      // adjacent query blocks per workgroup (fused path; 1 on the few-rows path)
+    int f_nwgq;      // workgroups along the query axis: ceil(f_nqblk / f_rbpw)
     int n_partials;  // slabs summed by the finalize kernel
     // workspace layout (byte offsets, each 256-byte aligned)
     size_t off_lse;      // float2 [B*H][rows_pad]            row maximum and log2 of the row sum
@@ -154,6 +156,8 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         if (hpb > H) hpb = H;
         p.f_hpg = hpb;
         p.f_hg = ceil_div(H, hpb);
+        p.f_rbpw = 1;
+        p.f_nwgq = 1;
         p.n_partials = p.f_hg;
         p.off_lse = p.off_ml = p.off_partial = 0;
         p.total = align256(sizeof(float) * (size_t)p.n_partials * B * Sk);
@@ -170,26 +174,36 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         p.f_qg = 8 / p.f_kg;
         p.f_tpw = ceil_div(tiles, p.f_kg);
         p.f_nqblk = ceil_div(p.q_rows, 32 * p.f_qg);
-        // Heads per workgroup: one workgroup is resident per compute unit, so the launch runs in
-        // generations of kComputeUnits workgroups, each as long as its heads plus about 0.6 of a
-        // head for starting and finishing.  Fewer heads per workgroup fill the last generation
-        // better (528 workgroups of 16 heads take three generations, 2112 of 4 take nine quarter-
-        // length ones) at the price of more starts and more partial slabs.
-        const long basef = (long)p.f_nqblk * B;
-        double best = 0.;
+        // Units per workgroup: a unit is one (query block, head); a workgroup takes f_rbpw adjacent
+        // query blocks times f_hpg heads.  One workgroup is resident per compute unit, so the launch
+        // runs in generations of kComputeUnits workgroups, each as long as its units plus about 0.7 of
+        // a unit for starting and finishing.  Fewer units per workgroup fill the last generation
+        // better (528 workgroups of 16 units take three generations, 2112 of 4 take nine quarter-
+        // length ones) at the price of more starts and more partial slabs; more units per workgroup
+        // save starts (512 workgroups of 16 units take two generations, 256 of 32 one).
         p.f_hpg = H;
-        for (int hpg = H; hpg >= 1; --hpg) {
-            const int hg = ceil_div(H, hpg);
-            if (ceil_div(H, hg) != hpg) continue;  // same grouping as a smaller hpg
-            const long gens = (basef * hg + kComputeUnits - 1) / kComputeUnits;
-            const double cost = (double)gens * (hpg + 0.6) + 0.01 * hg;
-            if (hpg == H || cost < best) {
-                best = cost;
-                p.f_hpg = hpg;
+        p.f_rbpw = 1;
+        double best = 0.;
+        bool first = true;
+        for (int rbpw = 1; rbpw <= 16 && (rbpw == 1 || rbpw <= p.f_nqblk); ++rbpw) {
+            const int nwgq = ceil_div(p.f_nqblk, rbpw);
+            if (ceil_div(p.f_nqblk, nwgq) != rbpw) continue;  // same grouping as a smaller rbpw
+            for (int hpg = H; hpg >= 1; --hpg) {
+                const int hg = ceil_div(H, hpg);
+                if (ceil_div(H, hg) != hpg) continue;  // same grouping as a smaller hpg
+                const long gens = ((long)nwgq * B * hg + kComputeUnits - 1) / kComputeUnits;
+                const double cost = (double)gens * ((double)hpg * rbpw + 0.7) + 0.01 * hg + 0.002 * rbpw;
+                if (first || cost < best) {
+                    first = false;
+                    best = cost;
+                    p.f_hpg = hpg;
+                    p.f_rbpw = rbpw;
+                }
             }
         }
         p.f_hg = ceil_div(H, p.f_hpg);
-        p.n_partials = p.f_hg * p.f_nqblk * p.f_qg;
+        p.f_nwgq = ceil_div(p.f_nqblk, p.f_rbpw);
+        p.n_partials = p.f_hg * p.f_nwgq * p.f_qg;
         size_t off = align256(sizeof(float) * (size_t)p.n_partials * B * Sk);
         p.off_lse = p.off_ml = p.off_partial = 0;
         p.total = off;

@@ -57,7 +57,8 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit():
 
     lib = _hip.lib()
     p = ctypes.c_void_p(4096)  # never dereferenced
-    st = (ctypes.c_int64 * 4)(64 * 16 * 2048 * 64, 2048 * 64, 64, 1)
-    assert lib.fcs_workspace_bytes(0, 64, 16, 2048, 2048, 64, -1) > (8 << 20)
-    assert lib.fcs_colsum_noncausal_f16_static(p, p, p, None, 64, 16, 2048, 64, st, st, 0.125, -1, None) == -7
+    # row statistics of the two-pass path: 8 bytes x 64 x 16 x 4096 rows alone exceed the static array
+    st = (ctypes.c_int64 * 4)(16 * 4096 * 64, 4096 * 64, 64, 1)
+    assert lib.fcs_workspace_bytes(0, 64, 16, 4096, 4096, 64, -1) > (8 << 20)
+    assert lib.fcs_colsum_noncausal_f16_static(p, p, p, None, 64, 16, 4096, 64, st, st, 0.125, -1, None) == -7
     assert "static scratch" in _hip.strerror(-7)
