@@ -192,7 +192,13 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
                 const int hg = ceil_div(H, hpg);
                 if (ceil_div(H, hg) != hpg) continue;  // same grouping as a smaller hpg
                 const long gens = ((long)nwgq * B * hg + kComputeUnits - 1) / kComputeUnits;
-                const double cost = (double)gens * ((double)hpg * rbpw + 0.7) + 0.01 * hg + 0.002 * rbpw;
+                double cost = (double)gens * ((double)hpg * rbpw + 0.7) + 0.01 * hg + 0.002 * rbpw;
+                // The 32 workgroups that an XCD runs at a time are neighbours in launch order: nwgq of
+                // them share a batch entry, i.e. one head's keys.  When the key heads they stream at
+                // the same time outgrow the XCD's 4 MiB L2, the re-reads of a head's keys by its row
+                // blocks miss (measured +6 % at B 256, S 1024 with 32 batch entries per XCD).
+                const long streams = (nwgq >= 32) ? 1 : (32 + nwgq - 1) / nwgq;
+                if (streams * (long)Sk * 128 > (5L << 19)) cost *= 1.08;
                 if (first || cost < best) {
                     first = false;
                     best = cost;
