@@ -182,8 +182,12 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
                         }
 #pragma unroll
                         for (int j = 0; j < 8; ++j) {  // fixed order: bit-reproducible
+                            // A split that pass 1 left unstabilised reports m = 0 and a sum of up to 2^120;
+                            // next to a stabilised split its weight 2^((0 - m) * c) alone underflows although
+                            // the product does not: the weights are applied as two square roots.
                             const float mn = fmaxf(mm, v[j].x);
-                            ll = ll * fast_exp2((mm - mn) * a.c) + v[j].y * fast_exp2((v[j].x - mn) * a.c);
+                            const float wa = fast_exp2((mm - mn) * (0.5f * a.c)), wb = fast_exp2((v[j].x - mn) * (0.5f * a.c));
+                            ll = (ll * wa) * wa + (v[j].y * wb) * wb;
                             mm = mn;
                         }
                     }

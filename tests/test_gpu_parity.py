@@ -790,6 +790,21 @@ def test_large_score_magnitudes(qs, ks, kw, bf16):
     assert rel <= max(RTOL, 1.5 * steps * abs(kw["scale"]) * ulp), (rel, steps, s_max)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("scale", [3.0, 2.0])
+def test_key_splits_of_mixed_kind_merge_without_underflow(scale, bf16):
+    """One query row against 3000 keys at scale 3: scale * score reaches 70 .. 90, so some key splits of
+    the row-statistics pass stay unstabilised (m = 0, sums up to 2^120) and others are stabilised
+    (m = 20 .. 30 in score units).  Merging them weighs the unstabilised sum by 2^((0 - m) * c), which
+    underflows on its own although the weighted sum does not; the means came out 2e-3 too large."""
+    g = torch.Generator().manual_seed(31 * 10000 + 191)
+    q = torch.randn((1, 8, 1, 64), generator=g)
+    k = torch.randn((1, 8, 3000, 64), generator=g)
+    q, k = (q.bfloat16(), k.bfloat16()) if bf16 else (q.half(), k.half())
+    out = _run(q, k, is_causal=True, scale=scale)
+    _assert_close(out.cpu().double(), _oracle(q.float(), k.float(), is_causal=True, scale=scale), f"mixed splits scale {scale}")
+
+
 # ---------------------------------------------------------------------------------------
 # one long point of each benchmark sweep (reference: benchmarks/benchmark_colsum.py:757-801)
 # ---------------------------------------------------------------------------------------
