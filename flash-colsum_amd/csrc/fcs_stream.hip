@@ -182,7 +182,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
                         }
 #pragma unroll
                         for (int j = 0; j < 8; ++j) {  // fixed order: bit-reproducible
-                            // A split that pass 1 left unstabilised reports m = 0 and a sum of up to 2^120;
+                            // A split that pass 1 left unstabilised reports m = 0 and a sum of up to 2^110;
                             // next to a stabilised split its weight 2^((0 - m) * c) alone underflows although
                             // the product does not: the weights are applied as two square roots.
                             const float mn = fmaxf(mm, v[j].x);
@@ -488,7 +488,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
 // exponentials are added up per ROW: register i of a lane keeps the running sum of its row over the
 // lane's keys for the whole split, and the 32 key lanes are added once at the end through LDS.
 // Common case: 2^(c * s) without max subtraction, exact while every row sum of the split stays inside
-// [2^-80, 2^120); a block that leaves that range redoes its keys in two more sweeps (row maxima, then
+// [2^-80, 2^110); a block that leaves that range redoes its keys in two more sweeps (row maxima, then
 // sums of 2^((s - m) * c), the maximum subtracted before the scale).  Writes (m, log2 l) per row, or
 // (m, l) per (split, row) when the keys are split; the column pass merges the splits.
 // PRE: see the column pass.  The common sweep runs on Q * c rounded to fp16 and accepts row sums below
@@ -721,7 +721,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
         const int qi = qw0 + nb * 32 + n;
         const int thr = a.causal ? min(a.k_past + qi, a.Sk - 1) : a.Sk - 1;  // last key this row sees
         has[nb] = (nst > 0) && (kc0 <= thr);
-        bad = bad || (has[nb] && !(lt[nb] >= 8.2718061e-25f && lt[nb] < (PRE ? kRowSumHiPre : 1.3292280e+36f)));
+        // ceiling 2^110 rather than 2^120: up to 512 key splits of a row are added up by the column pass
+        bad = bad || (has[nb] && !(lt[nb] >= 8.2718061e-25f && lt[nb] < (PRE ? kRowSumHiPre : 1.2980742e+33f)));
         m_row[nb] = has[nb] ? 0.f : kNegBig;  // an empty split must not set the merged maximum
         if (!has[nb]) lt[nb] = 0.f;
     }
