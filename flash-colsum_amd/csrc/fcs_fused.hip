@@ -22,7 +22,8 @@
 // The exponent is taken WITHOUT max subtraction while that is exact in fp32: every row
 // sum must land in [2^-80, 2^120).  If any row of the workgroup falls outside (or is not
 // finite) the block redoes that (head, row block) with the usual max-subtracted softmax.
-// A workgroup walks over its heads and writes one partial column-sum slab at the end;
+// A workgroup walks over its units (the heads of its head group times its row blocks, row blocks
+// innermost) and writes one partial column-sum slab at the end;
 // slabs have a single writer each and are added in index order by fcs_finalize_kernel.
 #include <hip/hip_runtime.h>
 #include <stdint.h>

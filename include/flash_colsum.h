@@ -84,7 +84,7 @@ int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *out
  * the library runs on holds until the process ends.  Has no counterpart in the reference.
  * Calls no hipMalloc / hipFree or any allocating routine.  Returns FCS_E_STATIC_LIMIT when
  * fcs_workspace_bytes(0, B, H, S, S, D, cls_n) exceeds FCS_STATIC_SCRATCH_BYTES (8 MiB: enough
- * for B=8 H=16 S=2048 D=64, which needs 4 MiB).  All calls on one GPU share that GPU's array:
+ * for B=8 H=16 S=2048 D=64, which needs 2 MiB).  All calls on one GPU share that GPU's array:
  * calls that overlap in time on one GPU (different streams or threads) race; calls on one
  * stream are ordered and safe.  Results are bit-identical to fcs_colsum_noncausal_f16. */
 int fcs_colsum_noncausal_f16_static(const void *q, const void *k, float *out, void *out_f16,
