@@ -576,7 +576,7 @@ def test_public_api_returns_fp16_like_the_reference():
 
 
 # ---------------------------------------------------------------------------------------
-# the binding stub of INTEGRATION.md, run as written
+# the binding stub shown to a maintainer of the reference (the integration notes at the repository root), run as written
 # ---------------------------------------------------------------------------------------
 def test_integration_stub_launchers():
     from flash_colsum import _hip

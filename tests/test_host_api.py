@@ -166,8 +166,8 @@ def test_missing_library_is_loud(monkeypatch, tmp_path):
 
 
 def integration_stub():
-    """The binding stub INTEGRATION.md shows to a maintainer of the reference, executed as written
-    (only the library's file name is replaced by its path in this tree)."""
+    """The binding stub that the integration notes at the repository root show to a maintainer of the
+    reference, executed as written (only the library's file name is replaced by its path in this tree)."""
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     blocks = re.findall(r"```python\n(.*?)```", text, flags=re.S)
     code = next(b for b in blocks if "_flash_colsum_batched" in b)
