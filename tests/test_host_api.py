@@ -85,6 +85,11 @@ def test_workspace_bytes():
     # never more than a few floats per (row, head) plus a few partial outputs: O(S), not O(S^2)
     assert wb(False, 8, 16, 2048, 2048, 64) < 64 << 20
     assert wb(True, 1, 32, 512, 65536, 128) < 64 << 20
+    # fused path: one slab per workgroup along the query axis.  B8 H16 S2048 runs as one generation of
+    # 256 workgroups (two row blocks x sixteen heads each): 32 slabs of (8, 2048) floats
+    assert wb(False, 8, 16, 2048, 2048, 64) == 32 * 8 * 2048 * 4
+    # B256 H16 S1024 (64-row blocks): eight row blocks per workgroup, two slabs of two query groups
+    assert wb(False, 256, 16, 1024, 1024, 64) == 2 * 2 * 256 * 1024 * 4
 
 
 def test_workspace_plan_over_random_shapes():
