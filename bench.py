@@ -37,6 +37,8 @@ WORKLOADS = {
     "noncausal_b2_h4_s512_d64": ((2, 4, 512, 64), (2, 4, 512, 64), dict(scale=0.125), False),
     "noncausal_b8_h16_s2048_d64": ((8, 16, 2048, 64), (8, 16, 2048, 64), dict(), True),
     "cls1_b32_h16_s577_d64": ((32, 16, 577, 64), (32, 16, 577, 64), dict(cls_len=1), False),
+    # a point of the reference's own batched sweep (benchmarks/benchmark_colsum.py:289-330), not a headline config
+    "noncausal_b256_h16_s1024_d64": ((256, 16, 1024, 64), (256, 16, 1024, 64), dict(), False),
     "causal_h32_q128_k4096_d128": ((1, 32, 128, 128), (1, 32, 4096, 128), dict(is_causal=True), False),
     "causal_h32_q128_k16384_d128": ((1, 32, 128, 128), (1, 32, 16384, 128), dict(is_causal=True), False),
     "causal_h32_q512_k65536_d128_peaky": ((1, 32, 512, 128), (1, 32, 65536, 128), dict(is_causal=True), False),
@@ -45,6 +47,7 @@ KERNELS_OF = {
     "noncausal_b2_h4_s512_d64": "fcs_fused_kernel<64,8,false,0,false> + fcs_finalize_kernel (one call)",
     "noncausal_b8_h16_s2048_d64": "fcs_fused_kernel<64,8,false,8,false> + fcs_finalize_kernel (one call; the fused kernel is >= 96 % of it)",
     "cls1_b32_h16_s577_d64": "fcs_fewrows_kernel<64,1> + fcs_finalize_kernel (one call)",
+    "noncausal_b256_h16_s1024_d64": "fcs_fused_kernel<64,8,false,4,false> + fcs_finalize_kernel (one call)",
     "causal_h32_q128_k4096_d128": "fcs_rowstream_kernel<128,1,4> + fcs_colstream_kernel<128,1,4> + fcs_finalize_kernel (one call)",
     "causal_h32_q128_k16384_d128": "fcs_rowstream_kernel<128,1,4> + fcs_colstream_kernel<128,1,4> + fcs_finalize_kernel (one call)",
     "causal_h32_q512_k65536_d128_peaky": "fcs_rowstream_kernel<128,2,8> + fcs_colstream_kernel<128,2,8> + fcs_finalize_kernel (one call)",
