@@ -790,6 +790,25 @@ def test_large_score_magnitudes(qs, ks, kw, bf16):
     assert rel <= max(RTOL, 1.5 * steps * abs(kw["scale"]) * ulp), (rel, steps, s_max)
 
 
+@pytest.mark.parametrize("qs,ks,kw", [
+    ((24, 4, 1024, 64), (24, 4, 1024, 64), {}),                    # 16 row blocks: whole groups of them
+    ((40, 6, 777, 64), (40, 6, 777, 64), {"cls_len": 500}),        # 8 blocks of 64 rows, the last one ragged
+    ((100, 2, 300, 64), (100, 2, 300, 64), {"scale": 0.3}),
+    ((16, 4, 1500, 64), (16, 4, 600, 64), {}),                     # S_q != S_k: 24 row blocks in uneven groups
+])
+def test_fused_path_with_several_row_blocks_per_workgroup(qs, ks, kw):
+    """Batches large enough that the launch plan gives a workgroup several adjacent row blocks per
+    head, including groups that the last workgroup along the query axis only fills in part."""
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(qs, generator=g).half()
+    k = torch.randn(ks, generator=g).half()
+    if qs[2] == ks[2]:
+        out, ref = _run(q, k, **kw), _oracle(q.float().cuda(), k.float().cuda(), **kw)
+    else:
+        out, ref = _run_ext(q, k, **kw), _oracle_ext(q.float().cuda(), k.float().cuda(), **kw)
+    _assert_close(out, ref, f"{qs} {ks} {kw}")
+
+
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("scale", [3.0, 2.0])
 def test_key_splits_of_mixed_kind_merge_without_underflow(scale, bf16):
