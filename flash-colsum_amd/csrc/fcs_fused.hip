@@ -38,7 +38,6 @@ namespace {
 constexpr float kSumLo = 8.2718061e-25f;  // 2^-80
 constexpr float kSumHi = 1.3292280e+36f;  // 2^120
 constexpr float kSumHiPre = 268435456.f;  // 2^28: ceiling of the pre-scaled variant (bounds its score rounding error)
-constexpr int kRedPitch = 40;             // floats per row of the wave-private transpose buffer
 
 #define FCS_GLDS16(gptr, lptr)                                                                \
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gptr), \
@@ -55,72 +54,72 @@ constexpr int kRedPitch = 40;             // floats per row of the wave-private 
 
 // LDS scratch of one workgroup for the row reductions
 struct RowRed {
-    float *red_w;  // wave-private [32][kRedPitch]
     float *part;   // [2][256]: per-wave row partials, double-buffered by reduction parity
     float *wv_w;   // wave-private [32]: the reduced (and post-processed) value of each row
     int parity;
 };
 
-// Sum of v[i] over the 32 lanes of each half-wave, for all sixteen i at once, in registers: a
-// reduce-scatter butterfly.  Each step adds the values of lanes 16, 8, 4, 2 apart while halving the
-// number of registers: which half a lane keeps is chosen by the lane-number bit of that step, so
-// after four steps a lane is left with ONE register, the total of
+// Sum (or maximum) of v[i] over the 32 lanes of each half-wave, for all sixteen i at once, in
+// registers: a reduce-scatter butterfly.  Each step combines the values of lanes 16, 8, 4, 2 apart
+// while halving the number of registers: which half a lane keeps is chosen by the lane-number bit
+// of that step, so after four steps a lane is left with ONE register, the total of
 //     i = 8 * bit4 + 4 * bit3 + 2 * bit2 + bit1        (bits of the lane number)
 // over 16 lanes; the last step (lanes 1 apart) completes it, both lanes of a pair hold the same
 // total.  In the accumulator layout that is row  16*bit4 + 8*bit3 + 4*g + 2*bit2 + bit1  (g = bit5).
-// 32 VALU instructions and no LDS traffic; the order of additions is fixed.
+// 32 VALU instructions and no LDS traffic; the order of operations is fixed.
 //   * 16 apart: v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even
-//     rows of its second, after which first + second is, in even rows, the sum of the first
+//     rows of its second, after which first (+) second is, in even rows, the total of the first
 //     register over the two rows and, in odd rows, that of the second register.
 //   * 8 and 4 apart: DPP row rotations; the bank mask (banks of 4 lanes) picks the lanes that keep
 //     the low or the high register of a pair, so no select is needed.
 //   * 2 and 1 apart: DPP quad permutations.
 // Inline assembly for the DPP forms: between a VALU write and a DPP read of the same register the
 // hardware wants two wait states, which the s_nop in front of every group provides.
-__device__ __forceinline__ float fold_lanes_sum(const float (&v)[16], int lane)
-{
-    float u[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        float x = v[i], y = v[i + 8];
-        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
-        u[i] = x + y;
+#define FCS_FOLD_LANES(NAME, OP, COMBINE)                                                                  \
+    __device__ __forceinline__ float NAME(const float (&v)[16], int lane)                                  \
+    {                                                                                                      \
+        float u[8];                                                                                        \
+        _Pragma("unroll") for (int i = 0; i < 8; ++i)                                                      \
+        {                                                                                                  \
+            float x = v[i], y = v[i + 8];                                                                  \
+            asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));        \
+            u[i] = COMBINE(x, y);                                                                          \
+        }                                                                                                  \
+        /* 8 apart: lanes with bit3 clear (banks 0, 1) keep u[j], the others u[j + 4] */                   \
+        asm volatile("s_nop 1\n\t" OP " %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0x3\n\t" OP            \
+                     " %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3\n\t" OP                             \
+                     " %2, %2, %2 row_ror:8 row_mask:0xf bank_mask:0x3\n\t" OP                             \
+                     " %3, %3, %3 row_ror:8 row_mask:0xf bank_mask:0x3\n\t" OP                             \
+                     " %0, %4, %4 row_ror:8 row_mask:0xf bank_mask:0xc\n\t" OP                             \
+                     " %1, %5, %5 row_ror:8 row_mask:0xf bank_mask:0xc\n\t" OP                             \
+                     " %2, %6, %6 row_ror:8 row_mask:0xf bank_mask:0xc\n\t" OP                             \
+                     " %3, %7, %7 row_ror:8 row_mask:0xf bank_mask:0xc"                                    \
+                     : "+v"(u[0]), "+v"(u[1]), "+v"(u[2]), "+v"(u[3])                                      \
+                     : "v"(u[4]), "v"(u[5]), "v"(u[6]), "v"(u[7]));                                        \
+        /* 4 apart (a rotation to the right by n hands lane i the value of lane i - n of its row): lanes  \
+           with bit2 clear (banks 0, 2) take their partner 4 lanes up, the others 4 lanes down */          \
+        asm volatile("s_nop 1\n\t" OP " %0, %0, %0 row_ror:12 row_mask:0xf bank_mask:0x5\n\t" OP           \
+                     " %1, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5\n\t" OP                            \
+                     " %0, %2, %2 row_ror:4 row_mask:0xf bank_mask:0xa\n\t" OP                             \
+                     " %1, %3, %3 row_ror:4 row_mask:0xf bank_mask:0xa"                                    \
+                     : "+v"(u[0]), "+v"(u[1])                                                              \
+                     : "v"(u[2]), "v"(u[3]));                                                              \
+        /* 2 apart: lanes with bit1 clear keep u[0] */                                                     \
+        const bool hi2 = (lane & 2) != 0;                                                                  \
+        float keep = hi2 ? u[1] : u[0], send = hi2 ? u[0] : u[1];                                          \
+        asm volatile("s_nop 1\n\t" OP " %0, %1, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"    \
+                     "s_nop 1\n\t" OP " %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf"         \
+                     : "+v"(keep)                                                                          \
+                     : "v"(send));                                                                         \
+        return keep;                                                                                       \
     }
-    // 8 apart: lanes with bit3 clear (banks 0, 1) keep u[j], the others u[j + 4]
-    asm volatile("s_nop 1\n\t"
-                 "v_add_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-                 "v_add_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-                 "v_add_f32_dpp %2, %2, %2 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-                 "v_add_f32_dpp %3, %3, %3 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-                 "v_add_f32_dpp %0, %4, %4 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                 "v_add_f32_dpp %1, %5, %5 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                 "v_add_f32_dpp %2, %6, %6 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                 "v_add_f32_dpp %3, %7, %7 row_ror:8 row_mask:0xf bank_mask:0xc"
-                 : "+v"(u[0]), "+v"(u[1]), "+v"(u[2]), "+v"(u[3])
-                 : "v"(u[4]), "v"(u[5]), "v"(u[6]), "v"(u[7]));
-    // 4 apart (a rotation to the right by n hands lane i the value of lane i - n of its row): lanes with
-    // bit2 clear (banks 0, 2) take their partner 4 lanes up, the others 4 lanes down
-    asm volatile("s_nop 1\n\t"
-                 "v_add_f32_dpp %0, %0, %0 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
-                 "v_add_f32_dpp %1, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
-                 "v_add_f32_dpp %0, %2, %2 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
-                 "v_add_f32_dpp %1, %3, %3 row_ror:4 row_mask:0xf bank_mask:0xa"
-                 : "+v"(u[0]), "+v"(u[1])
-                 : "v"(u[2]), "v"(u[3]));
-    // 2 apart: lanes with bit1 clear keep u[0]
-    const bool hi2 = (lane & 2) != 0;
-    float keep = hi2 ? u[1] : u[0], send = hi2 ? u[0] : u[1];
-    asm volatile("s_nop 1\n\t"
-                 "v_add_f32_dpp %0, %1, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
-                 "s_nop 1\n\t"
-                 "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf"
-                 : "+v"(keep)
-                 : "v"(send));
-    return keep;
-}
+__device__ __forceinline__ float fcs_add2(float x, float y) { return x + y; }
+FCS_FOLD_LANES(fold_lanes_sum, "v_add_f32_dpp", fcs_add2)
+FCS_FOLD_LANES(fold_lanes_max, "v_max_f32_dpp", fmaxf)
+#undef FCS_FOLD_LANES
 
 // Reduces v[16] (v[i] belongs to row acc_row(i, g) of the wave's 32 rows) over the 32 lanes of
-// each half-wave (sums: in registers, fold_lanes_sum; maxima: a transpose through LDS) and over
+// each half-wave (in registers: fold_lanes_sum / fold_lanes_max) and over
 // the key-group waves of the same query group: sum, or max if MAX.
 // `post(row_in_block, total)` maps the total to what is left in rr.wv_w[row] for the lanes to
 // read back.  Returns (sum only) whether any row total of the WORKGROUP is outside
@@ -129,27 +128,11 @@ template <bool MAX, typename Post>
 __device__ __forceinline__ bool reduce_rows(const float (&v)[16], RowRed &rr, int kg_n, int qg, int kg, int lane, Post post,
                                             const float sum_hi = kSumHi)
 {
-    const int n = lane & 31, g = lane >> 5;
+    const int g = lane >> 5;
     const int row = lane >> 1, half = lane & 1;  // after the barrier lane L works on row L / 2
-    int row_w = row;                             // the row whose total over this wave's keys the lane holds before it
-    float s;
-    if (!MAX) {
-        s = fold_lanes_sum(v, lane);
-        row_w = 16 * ((lane >> 4) & 1) + 8 * ((lane >> 3) & 1) + 4 * g + 2 * ((lane >> 2) & 1) + ((lane >> 1) & 1);
-    } else {
-        // maxima (rare path): transpose through the wave's own LDS block (LDS executes a wave's accesses in order)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) rr.red_w[acc_row(i, g) * kRedPitch + n] = v[i];
-        __builtin_amdgcn_wave_barrier();
-        const floatx4 *src = reinterpret_cast<const floatx4 *>(rr.red_w + row * kRedPitch);
-        floatx4 x[4];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) x[c] = src[2 * c + half];
-        s = x[0][0];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) s = fmaxf(fmaxf(fmaxf(s, x[c][0]), fmaxf(x[c][1], x[c][2])), x[c][3]);
-        s = fmaxf(s, dpp_get<kDppXor1>(s));
-    }
+    // the row whose total over this wave's keys the lane holds before it
+    const int row_w = 16 * ((lane >> 4) & 1) + 8 * ((lane >> 3) & 1) + 4 * g + 2 * ((lane >> 2) & 1) + ((lane >> 1) & 1);
+    const float s = MAX ? fold_lanes_max(v, lane) : fold_lanes_sum(v, lane);
     // waves: one partial per (row, key group), dense so that 256 floats cover the workgroup
     float *part = rr.part + (rr.parity & 1) * 256;
     rr.parity ^= 1;
@@ -226,7 +209,6 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     constexpr int SLOT_BYTES = NT * 1024;  // one item: NT pieces x 64 lanes x 16 bytes
     constexpr bool STATIC_SLOTS = (ITEMS % NS == 0);  // then item j of every head sits in slot j % NS
     __shared__ __attribute__((aligned(16))) char ring[8 * NS * SLOT_BYTES];
-    __shared__ __attribute__((aligned(16))) float red[8 * 32 * kRedPitch];
     __shared__ __attribute__((aligned(16))) float part[2 * 256];
     __shared__ __attribute__((aligned(16))) float wv[8 * 32];
     constexpr int PQG = PRE ? 8 / PRE : 1;  // query groups of the pre-scaled variant
@@ -257,7 +239,6 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     const int kbase = kg * TPW * 32;        // first key of this wave
 
     RowRed rr;
-    rr.red_w = red + wave * (32 * kRedPitch);
     rr.part = part;
     rr.wv_w = wv + wave * 32;
     rr.parity = 0;
