@@ -203,11 +203,15 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     static_assert(D == 64, "the fused path is laid out for 64-wide heads");
     static_assert(!(PRE && BF), "the pre-scaled variant rounds Q*c to fp16; bf16 would be too coarse");
     constexpr int NT = D / 16;             // MFMA steps (and 16-byte pieces per lane) per operand tile
-    constexpr int NS = 3;                  // ring slots per wave
-    constexpr int AHEAD = NS - 1;          // items in flight ahead of the one being consumed
+    // KRING (whole-tile pre-scaled variants whose tile count is a multiple of four): the ring holds key
+    // tiles only, in four slots.  The Q item of those variants is a plain load that needs no slot, so
+    // key tile k of every unit sits in slot k % 4 and three key tiles are in flight ahead of the one
+    // being used instead of two.
+    constexpr bool KRING = PRE && !RAGGED && TPW % 4 == 0;
+    constexpr int NS = KRING ? 4 : 3;      // ring slots per wave
     constexpr int ITEMS = TPW + 1;         // per (head, row block): the Q tile, then TPW key tiles
     constexpr int SLOT_BYTES = NT * 1024;  // one item: NT pieces x 64 lanes x 16 bytes
-    constexpr bool STATIC_SLOTS = (ITEMS % NS == 0);  // then item j of every head sits in slot j % NS
+    constexpr bool STATIC_SLOTS = KRING || (ITEMS % NS == 0);  // then an item's slot is a compile-time value
     __shared__ __attribute__((aligned(16))) char ring[8 * NS * SLOT_BYTES];
     __shared__ __attribute__((aligned(16))) float part[2 * 256];
     __shared__ __attribute__((aligned(16))) float wv[8 * 32];
@@ -315,7 +319,8 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             const uint32_t ta0 = take_addr[0], ta1 = take_addr[1], ta2 = take_addr[2], ta3 = take_addr[3];
             if (slot == 0) FCS_TAKE_ASM(0);
             else if (slot == 1) FCS_TAKE_ASM(4096);
-            else FCS_TAKE_ASM(8192);
+            else if (slot == 2) FCS_TAKE_ASM(8192);
+            else FCS_TAKE_ASM(12288);
         } else {
             const uint32_t off = (uint32_t)(slot * SLOT_BYTES);
             const uint32_t ta0 = take_addr[0] + off, ta1 = take_addr[1] + off, ta2 = take_addr[2] + off, ta3 = take_addr[3] + off;
@@ -475,8 +480,22 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     };
 
     half8 qf[NT], kf[2][NT];
+    // item of key tile r counted from the current unit's first (r >= TPW: the next unit's), and the
+    // step at which the next unit's Q rows are requested (KRING)
+    auto ktile_item = [&](int r) { return r < TPW ? 1 + r : ITEMS + 1 + (r - TPW); };
+    constexpr int TQ = TPW - 2;
+    if (KRING) {
+        // same order of requests as at the end of every unit: key tiles 0 .. NS-3, the Q rows, key tiles
+        // NS-2 and NS-1, so that the counted waits below hold for the first unit too
 #pragma unroll
-    for (int i = 0; i < NS; ++i) fetch_pos(i, i);
+        for (int r = 0; r < NS - 2; ++r) fetch_pos(ktile_item(r), r);
+        fetch_pos(0, 0);
+        fetch_pos(ktile_item(NS - 2), NS - 2);
+        fetch_pos(ktile_item(NS - 1), NS - 1);
+    } else {
+#pragma unroll
+        for (int i = 0; i < NS; ++i) fetch_pos(i, i);
+    }
     if (PRE) {
         q_publish(0);
         __syncthreads();
@@ -496,8 +515,14 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             FCS_WAIT_VM(2 * NT);
             take_issue(slot_of(0), qf);
         }
-        FCS_WAIT_VM(1 * NT);
-        take_issue(slot_of(1), kf[0]);
+        if (KRING) {
+            // key tile 0 was requested NS steps ago; behind it: NS - 1 key tiles and the Q rows
+            FCS_WAIT_VM((NS - 1) * NT + 1);
+            take_issue(0, kf[0]);
+        } else {
+            FCS_WAIT_VM(1 * NT);
+            take_issue(slot_of(1), kf[0]);
+        }
         floatx16 acc[TPW];
         float rs[16];
 #pragma unroll
@@ -542,6 +567,21 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             else asm volatile("s_setprio 0");
             // the operands of this tile were read back during the previous step: they have landed,
             // their ring slots are free again and take the look-ahead fetches
+            if (KRING) {
+                if (t == 0) take_wait(qf);
+                take_wait(kf[t & 1]);
+                // the slot of key tile t is free: it takes key tile t + NS; the next unit's Q rows are
+                // requested at step TQ, before that step's key tile
+                if (t == TQ) fetch_pos(ITEMS, 0);
+                fetch_pos(ktile_item(t + NS), t % NS);
+                // key tile t + 1 has landed once only what was requested behind it is outstanding: the
+                // NS - 1 key tiles of steps t + 2 - NS .. t, and the Q rows if their step is among those
+                constexpr int TQ_PREV = TQ - TPW;  // the previous unit's request, seen from this unit
+                const bool q_behind = (TQ >= t + 2 - NS && TQ <= t) || (TQ_PREV >= t + 2 - NS && TQ_PREV <= t);
+                if (q_behind) FCS_WAIT_VM((NS - 1) * NT + 1);
+                else FCS_WAIT_VM((NS - 1) * NT);
+                if (t + 1 < TPW) take_issue((t + 1) % NS, kf[(t + 1) & 1]);
+            } else {
             if (t == 0) {
                 take_wait(qf);
                 take_wait(kf[0]);
@@ -559,6 +599,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             if (item_vm(t + 3) + item_vm(t + 4) == 2 * NT) FCS_WAIT_VM(2 * NT);
             else FCS_WAIT_VM(NT + 1);
             if (t + 1 < TPW) take_issue(slot_of(2 + t), kf[(t + 1) & 1]);
+            }
             floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int tt = 0; tt < NT; ++tt) c = mfma16<BF>(qf[tt], kf[t & 1][tt], c);
