@@ -203,11 +203,11 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     static_assert(D == 64, "the fused path is laid out for 64-wide heads");
     static_assert(!(PRE && BF), "the pre-scaled variant rounds Q*c to fp16; bf16 would be too coarse");
     constexpr int NT = D / 16;             // MFMA steps (and 16-byte pieces per lane) per operand tile
-    // KRING (whole-tile pre-scaled variants whose tile count is a multiple of four): the ring holds key
+    // KRING (pre-scaled variants whose tile count is a multiple of four): the ring holds key
     // tiles only, in four slots.  The Q item of those variants is a plain load that needs no slot, so
     // key tile k of every unit sits in slot k % 4 and three key tiles are in flight ahead of the one
     // being used instead of two.
-    constexpr bool KRING = PRE && !RAGGED && TPW % 4 == 0;
+    constexpr bool KRING = PRE && TPW % 4 == 0;
     constexpr int NS = KRING ? 4 : 3;      // ring slots per wave
     constexpr int ITEMS = TPW + 1;         // per (head, row block): the Q tile, then TPW key tiles
     constexpr int SLOT_BYTES = NT * 1024;  // one item: NT pieces x 64 lanes x 16 bytes
@@ -413,9 +413,10 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     };
     auto fetch_pos = [&](int j_ahead, int slot) {
         if (RAGGED) {
-            // One wave-uniform decision per tile: a tile that lies wholly inside its tensor and has
-            // dense rows takes the cheap whole-tile form; only tiles that touch the end (or strided
-            // rows) pay for per-lane row clamping.
+            // One wave-uniform decision per tile: a tile that lies wholly inside its tensor takes a
+            // cheap form (dense rows: the whole-tile form; any other row pitch, e.g. (B,S,H,D) storage:
+            // the same lane offsets with the tile base advanced by eight rows per instruction); only
+            // tiles that touch the end pay for per-lane row clamping.
             const int ua = j_ahead / ITEMS;
             const int j = j_ahead % ITEMS;
             const bool is_q = (j == 0);
@@ -430,6 +431,15 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 const char *tile = slice + (size_t)first_row * (D * 2);
 #pragma unroll
                 for (int tt = 0; tt < NT; ++tt) fetch_piece(true, tile, row_b, dense_voff, 0, 0, slot, tt);
+            } else if (first_row + 32 <= n_rows) {
+                const char *tile = slice + (size_t)first_row * row_b;
+                char *dst = my_ring + slot * SLOT_BYTES;
+#pragma unroll
+                for (int tt = 0; tt < NT; ++tt) {
+                    uint32_t vo = is_q ? q_voff[tt & 1] : k_voff[tt & 1];
+                    FCS_OPAQUE_V(vo);
+                    FCS_GLDS16(tile + (size_t)(tt * 8) * row_b + vo, dst + tt * 1024);
+                }
             } else {
 #pragma unroll
                 for (int tt = 0; tt < NT; ++tt) fetch_piece(false, slice, row_b, dense_voff, first_row, n_rows, slot, tt);
