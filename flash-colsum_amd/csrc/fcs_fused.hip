@@ -347,7 +347,9 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     //     instructions at every wait is a compile-time constant.
     // PRE: the Q item of a head is not a tile in the ring but this wave's 32 / PRE rows of its query
     // group's raw tile (512 B or 1 KB), one ordinary 8- or 16-byte load per lane; the wave scales
-    // them and publishes them in `qshare`.
+    // them and publishes them in `qshare`.  KRING: that item then takes no slot number either; key
+    // tile k of every unit lives in slot k % 4, key tile k + 4 is fetched when tile k has been read
+    // back, and the next unit's Q rows are requested at step TPW - 2.
     // raw Q rows of the pre-scaled variant: written by an asynchronous load and read after a hand-placed
     // wait, so the variable the load names must be the one the wait names (no copies in between)
     typedef uint32_t qraw_t __attribute__((ext_vector_type(PRE == 8 ? 2 : 4)));
