@@ -241,6 +241,14 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     const int rb_first = qwg * a.f_rbpw, rb_n = min(a.f_rbpw, a.f_nqblk - rb_first);
     const int n_units = rb_n * n_heads;
     const int kbase = kg * TPW * 32;        // first key of this wave
+    // Ragged kernel: key tile t of this wave nominally holds keys [kbase + 32 t, kbase + 32 t + 32).
+    // A tile that would reach past the last key is moved back so that it ends there (every row it
+    // fetches exists; S_k >= 32 on this path): MFMA column n of tile t is key tile_first(t) + n, and
+    // the columns that repeat keys of the tile before it, n < kbase + 32 t + 32 - S_k, count for
+    // nothing.  For a lane that is t > tmax_lane.  No branch and no per-lane address arithmetic
+    // depends on where the keys end.
+    auto tile_first = [&](int t) { return RAGGED ? min(kbase + t * 32, a.Sk - 32) : kbase + t * 32; };
+    int tmax_lane = RAGGED ? (n + a.Sk - 32 - kbase) >> 5 : TPW;  // arithmetic shift: floor, also when negative
 
     RowRed rr;
     rr.part = part;
@@ -253,49 +261,66 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // LDS.  To keep the later operand reads (32 lanes, 128 B apart) off each other's banks
     // the pieces of a row are stored XOR-swizzled: position p of row r holds piece
     // p ^ ((r >> 1) & 7).  The swizzle only depends on the parity of the instruction index.
-    int lrow = lane >> 3;  // row within the 8 rows of one DMA instruction
-    uint32_t piece_b[2];   // byte offset in its row of the piece this lane fetches (even / odd instruction)
-#pragma unroll
-    for (int par = 0; par < 2; ++par) piece_b[par] = (uint32_t)(((lane & 7) ^ ((par * 4 + (lane >> 4)) & 7)) * 16);
+    // Lane L's part of one DMA instruction: its row within the instruction's 8 rows, and the byte
+    // offset in that row of the piece it fetches (instructions of even / odd index differ).
+    auto dma_row = [](int l) { return l >> 3; };
+    auto dma_piece_b = [](int l, int par) { return (uint32_t)(((l & 7) ^ ((par * 4 + (l >> 4)) & 7)) * 16); };
     // row pitch in bytes; a compile-time constant in the non-ragged kernel (rows are dense there)
     const uint32_t q_row_b = RAGGED ? (uint32_t)a.qs_s * 2u : (uint32_t)(D * 2), k_row_b = RAGGED ? (uint32_t)a.ks_s * 2u : (uint32_t)(D * 2);
-    uint32_t dense_voff[2] = {lrow * (uint32_t)(D * 2) + piece_b[0], lrow * (uint32_t)(D * 2) + piece_b[1]};  // ragged kernel's whole tiles
-    uint32_t q_voff[2] = {lrow * q_row_b + piece_b[0], lrow * q_row_b + piece_b[1]};
-    uint32_t k_voff[2] = {lrow * k_row_b + piece_b[0], lrow * k_row_b + piece_b[1]};
+    // Lane offsets from a tile's first row to this lane's piece.  Whole-tile kernel: rows are dense,
+    // so instruction tt reads exactly 1 KB behind instruction tt - 2 and the offsets of instructions
+    // 0 and 1 serve all four.  Ragged kernel (key tiles): rows have any pitch, so each instruction has
+    // its own offset; it is stored less tt KB, because the instruction's immediate offset (which the
+    // hardware adds to the LDS address AND the global address) supplies tt KB again.  (Never negative:
+    // a row is at least 128 bytes.)
+    auto ragged_voff = [&](int l, uint32_t row_b, int tt) {
+        return (uint32_t)(dma_row(l) + 8 * tt) * row_b + dma_piece_b(l, tt & 1) - (uint32_t)(tt * 1024);
+    };
+    constexpr int NVOFF = RAGGED ? NT : 2;
+    uint32_t q_voff[2] = {dma_row(lane) * q_row_b + dma_piece_b(lane, 0), dma_row(lane) * q_row_b + dma_piece_b(lane, 1)};
+    uint32_t k_voff[NVOFF];
+#pragma unroll
+    for (int i = 0; i < NVOFF; ++i) k_voff[i] = RAGGED ? ragged_voff(lane, k_row_b, i) : dma_row(lane) * k_row_b + dma_piece_b(lane, i);
     // start of this batch entry's Q / K (head 0, row 0), and the same advanced to this wave's first
     // row.  Only the whole-tile kernel addresses through the latter: there every row it names
-    // exists.  The ragged kernel and the rare slow path clamp ABSOLUTE row numbers instead, because
-    // a wave's rows (and whole tiles of them) may lie past the end of the tensor.
+    // exists.  The ragged kernel works from ABSOLUTE row numbers instead (Q rows clamped to the last
+    // one, key tiles moved back to end at the last key), because a wave's rows (and whole tiles of
+    // them) may lie past the end of the tensor.
     const char *q_batch = reinterpret_cast<const char *>(a.q + (int64_t)b * a.qs_b);
     const char *k_batch = reinterpret_cast<const char *>(a.k + (int64_t)b * a.ks_b);
     const char *k_b = k_batch + (int64_t)min(kbase, a.Sk - 1) * k_row_b;
     const int64_t q_head_b = a.qs_h * 2, k_head_b = a.ks_h * 2;
     char *my_ring = ring + wave * (NS * SLOT_BYTES);
 
-    // DMA instruction `tt` (of NT) of a tile: its rows [8*tt, 8*tt + 8) go to ring slot `slot`.
-    // Whole-tile kernel: `tile` (wave-uniform) is the tile's first row.  Ragged kernel: `tile` is
-    // row 0 of the head's slice, the tile starts at row `first_row` of its `n_rows`, and rows past
-    // the end are replaced by the last real row (the consumer masks or ignores them).  No branch
-    // either way: a taken branch costs a wave far more than the few address instructions it would skip.
-    auto fetch_piece = [&](bool whole_tile, const char *tile, uint32_t row_b, uint32_t (&voff)[2], int first_row, int n_rows,
-                           int slot, int tt) {
+    // DMA instruction `tt` (of NT) of a whole tile with dense rows, first row at `tile` (wave-uniform):
+    // its rows [8*tt, 8*tt + 8) go to ring slot `slot`.  Instruction tt reads 1 KB further in memory
+    // and writes 1 KB further in the slot, which is exactly what the immediate offset does; base
+    // pointer, lane offset and LDS base are shared by the four pieces.
+    auto fetch_piece_at = [&](const char *tile, uint32_t vo, int slot, int tt) {
         char *dst = my_ring + slot * SLOT_BYTES;
-        if (whole_tile) {
-            // every tile is whole and its rows are dense: instruction tt reads 1 KB further in
-            // memory and writes 1 KB further in the slot, which is exactly what the immediate
-            // offset does; base pointer, lane offset and LDS base are shared by the four pieces
-            static_assert(NT == 4, "offsets below");
-            FCS_OPAQUE_V(voff[tt & 1]);
-            const char *src = tile + voff[tt & 1];
-            if (tt == 0) FCS_GLDS16_OFF(src, dst, 0);
-            else if (tt == 1) FCS_GLDS16_OFF(src, dst, 1024);
-            else if (tt == 2) FCS_GLDS16_OFF(src, dst, 2048);
-            else FCS_GLDS16_OFF(src, dst, 3072);
-        } else {
-            FCS_OPAQUE_V(lrow);
-            FCS_OPAQUE_V(piece_b[tt & 1]);
-            const uint32_t row = (uint32_t)min(first_row + tt * 8 + lrow, n_rows - 1);
-            FCS_GLDS16(tile + ((size_t)row * row_b + piece_b[tt & 1]), dst + tt * 1024);
+        static_assert(NT == 4, "offsets below");
+        const char *src = tile + vo;
+        if (tt == 0) FCS_GLDS16_OFF(src, dst, 0);
+        else if (tt == 1) FCS_GLDS16_OFF(src, dst, 1024);
+        else if (tt == 2) FCS_GLDS16_OFF(src, dst, 2048);
+        else FCS_GLDS16_OFF(src, dst, 3072);
+    };
+    auto fetch_piece = [&](const char *tile, auto &voff, int slot, int tt) {
+        FCS_OPAQUE_V(voff[tt & 1]);
+        fetch_piece_at(tile, voff[tt & 1], slot, tt);
+    };
+    // Ragged kernel, the Q tile at rows [first_row, first_row + 32) of a slice of `n_rows` rows of any
+    // pitch (once per unit): each lane clamps its row to the last real one (repeated rows carry
+    // weight 0 in the column sums).  No branch: a taken branch costs a wave far more than these few
+    // address instructions.
+    auto fetch_ragged_q = [&](const char *slice, uint32_t row_b, int first_row, int n_rows, int slot) {
+        char *dst = my_ring + slot * SLOT_BYTES;
+        int l = lane;
+        FCS_OPAQUE_V(l);
+#pragma unroll
+        for (int tt = 0; tt < NT; ++tt) {
+            const uint32_t row = (uint32_t)min(first_row + tt * 8 + dma_row(l), n_rows - 1);
+            FCS_GLDS16(slice + ((size_t)row * row_b + dma_piece_b(l, tt & 1)), dst + tt * 1024);
         }
     };
     // Read a ring slot back as an MFMA operand: lane (n, g) takes, for step tt, piece 2*tt + g of
@@ -409,42 +434,23 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 else asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qraw) : "v"(src) : "memory");
             }
         } else if (j == 0)
-            fetch_piece(true, u_qtile[ua], q_row_b, q_voff, 0, 0, slot, tt);
+            fetch_piece(u_qtile[ua], q_voff, slot, tt);
         else
-            fetch_piece(true, k_b + k_off[ua] + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_row_b, k_voff, 0, 0, slot, tt);
+            fetch_piece(k_b + k_off[ua] + (size_t)((uint32_t)((j - 1) * 32) * k_row_b), k_voff, slot, tt);
     };
     auto fetch_pos = [&](int j_ahead, int slot) {
         if (RAGGED) {
-            // One wave-uniform decision per tile: a tile that lies wholly inside its tensor takes a
-            // cheap form (dense rows: the whole-tile form; any other row pitch, e.g. (B,S,H,D) storage:
-            // the same lane offsets with the tile base advanced by eight rows per instruction); only
-            // tiles that touch the end pay for per-lane row clamping.
             const int ua = j_ahead / ITEMS;
             const int j = j_ahead % ITEMS;
-            const bool is_q = (j == 0);
-            if (PRE && is_q) {  // the Q item of the pre-scaled variant is a plain load, not a tile
-                fetch_pos_piece(j_ahead, slot, 0);
-                return;
-            }
-            const char *slice = is_q ? u_qhead[ua] : k_batch + k_off[ua];
-            const int first_row = is_q ? u_qfirst[ua] : kbase + (j - 1) * 32, n_rows = is_q ? a.Sq : a.Sk;
-            const uint32_t row_b = is_q ? q_row_b : k_row_b;
-            if (first_row + 32 <= n_rows && row_b == (uint32_t)(D * 2)) {
-                const char *tile = slice + (size_t)first_row * (D * 2);
-#pragma unroll
-                for (int tt = 0; tt < NT; ++tt) fetch_piece(true, tile, row_b, dense_voff, 0, 0, slot, tt);
-            } else if (first_row + 32 <= n_rows) {
-                const char *tile = slice + (size_t)first_row * row_b;
-                char *dst = my_ring + slot * SLOT_BYTES;
+            if (j == 0 && PRE) fetch_pos_piece(j_ahead, slot, 0);  // the Q item of the pre-scaled variant is a plain load, not a tile
+            else if (j == 0) fetch_ragged_q(u_qhead[ua], q_row_b, u_qfirst[ua], a.Sq, slot);
+            else {
+                const char *tile = k_batch + k_off[ua] + (size_t)tile_first(j - 1) * k_row_b;
 #pragma unroll
                 for (int tt = 0; tt < NT; ++tt) {
-                    uint32_t vo = is_q ? q_voff[tt & 1] : k_voff[tt & 1];
-                    FCS_OPAQUE_V(vo);
-                    FCS_GLDS16(tile + (size_t)(tt * 8) * row_b + vo, dst + tt * 1024);
+                    FCS_OPAQUE_V(k_voff[tt % NVOFF]);
+                    fetch_piece_at(tile, k_voff[tt % NVOFF], slot, tt);
                 }
-            } else {
-#pragma unroll
-                for (int tt = 0; tt < NT; ++tt) fetch_piece(false, slice, row_b, dense_voff, first_row, n_rows, slot, tt);
             }
         } else {
 #pragma unroll
@@ -542,25 +548,18 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 
         // e = 2^(c*s) for tile t, in place, and its contribution to the row sums
         auto exp_tile = [&](int t) {
-            // ragged: a key past the end gets the bias -inf, so its exponential is 0; the bias rides
-            // on the scale multiply (one FMA) instead of costing a select per score
-            const float bias = (!RAGGED || (kbase + t * 32 + n) < a.Sk) ? 0.f : -INFINITY;
-            if (PRE && RAGGED && kbase + t * 32 + 31 >= a.Sk) {
-                // pre-scaled scores have no multiply to carry the bias: only a tile that reaches
-                // past the last key (wave-uniform test) pays an add per score
+            // ragged: a column that counts for nothing (see tile_first) gets the bias -inf, so its
+            // exponential is 0; the bias rides on the scale multiply (one FMA).  Pre-scaled scores have
+            // no multiply to carry it: there the column's exponentials (finite: they repeat real keys)
+            // enter the row sums with weight 0 (an FMA in place of the add).
+            const bool counts = !RAGGED || t <= tmax_lane;
+            const float bias = counts ? 0.f : -INFINITY, one = counts ? 1.f : 0.f;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float e = fast_exp2(acc[t][i] + bias);
-                    acc[t][i] = e;
-                    rs[i] += e;
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float e = fast_exp2(PRE ? acc[t][i] : (RAGGED ? fmaf(acc[t][i], a.c, bias) : acc[t][i] * a.c));
-                    acc[t][i] = e;
-                    rs[i] += e;
-                }
+            for (int i = 0; i < 16; ++i) {
+                const float e = fast_exp2(PRE ? acc[t][i] : (RAGGED ? fmaf(acc[t][i], a.c, bias) : acc[t][i] * a.c));
+                acc[t][i] = e;
+                if (PRE && RAGGED) rs[i] = fmaf(e, one, rs[i]);
+                else rs[i] += e;
             }
             // pinned here: otherwise the optimiser sinks every exponent below the last MFMA
             asm volatile("" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]), "+v"(rs[4]), "+v"(rs[5]), "+v"(rs[6]),
@@ -651,6 +650,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             int lane_s = lane;
             FCS_OPAQUE_V(lane_s);
             const int n_s = lane_s & 31, g_s = lane_s >> 5;
+            const int tmax_s = (n_s + a.Sk - 32 - kbase) >> 5;  // tmax_lane again
             const _Float16 *qp = reinterpret_cast<const _Float16 *>(q_batch + (int64_t)h * q_head_b) +
                                  (int64_t)min(q_first + n_s, a.Sq - 1) * a.qs_s + g_s * 8;
             const _Float16 *kp = reinterpret_cast<const _Float16 *>(k_batch + (int64_t)kv_head(h, a.kv_group, a.kv_magic) * k_head_b) + g_s * 8;
@@ -662,7 +662,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             }
             auto score_tile = [&](int t) {
                 half8 ks[NT];
-                const int krow = min(kbase + t * 32 + n_s, a.Sk - 1);
+                const int krow = RAGGED ? tile_first(t) + n_s : kbase + t * 32 + n_s;
 #pragma unroll
                 for (int tt = 0; tt < NT; ++tt) ks[tt] = load8(kp + (int64_t)krow * a.ks_s + tt * 16);
                 floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -676,7 +676,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 #pragma unroll 1
             for (int t = 0; t < TPW; ++t) {
                 const floatx16 c = score_tile(t);
-                const bool real = (kbase + t * 32 + n_s) < a.Sk;
+                const bool real = !RAGGED || t <= tmax_s;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) v16[i] = fmaxf(v16[i], real ? c[i] : kNegBig);
             }
@@ -693,7 +693,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 #pragma unroll 1
             for (int t = 0; t < TPW; ++t) {
                 const floatx16 c = score_tile(t);
-                const bool real = (kbase + t * 32 + n_s) < a.Sk;
+                const bool real = !RAGGED || t <= tmax_s;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) v16[i] += real ? fast_exp2((c[i] - rmax[i]) * a.c) : 0.f;
             }
@@ -709,7 +709,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 #pragma unroll 1
             for (int t = 0; t < TPW; ++t) {
                 const floatx16 c = score_tile(t);
-                const bool real = (kbase + t * 32 + n_s) < a.Sk;
+                const bool real = !RAGGED || t <= tmax_s;
                 float sum = 0.f;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) sum = fmaf(real ? fast_exp2((c[i] - rmax[i]) * a.c) : 0.f, v16[i], sum);
@@ -731,8 +731,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
         const float v = col_acc[t] + __shfl_xor(col_acc[t], 32);
-        const int key = kbase + t * 32 + n;
-        if (g == 0 && key < a.Sk) dst[key] = v;
+        if (g == 0 && t <= tmax_lane) dst[tile_first(t) + n] = v;
     }
 }
 
@@ -776,6 +775,7 @@ static bool launch_fused_t(const Plan &p, const Args &a, hipStream_t st)
 
 hipError_t launch_fused(const Plan &p, const Args &a, hipStream_t st)
 {
+    if (p.Sk < 32) return hipErrorInvalidValue;  // the ragged kernel fetches whole key tiles that end at the last key
     if (!(p.bf16 ? launch_fused_t<true>(p, a, st) : launch_fused_t<false>(p, a, st))) return hipErrorInvalidValue;
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

@@ -166,7 +166,8 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
 
     // ---- fused path
     p.n_partials = p.c_groups;
-    if (!causal && Sk <= kFusedMaxKeys && D == 64) {
+    // (at least one whole key tile: the kernel moves a tile that reaches past the last key back to end there)
+    if (!causal && Sk >= 32 && Sk <= kFusedMaxKeys && D == 64) {
         p.fused = 1;
         const int tiles = ceil_div(Sk, 32);
         p.f_kg = 1;
