@@ -809,6 +809,29 @@ def test_fused_path_with_several_row_blocks_per_workgroup(qs, ks, kw):
     _assert_close(out, ref, f"{qs} {ks} {kw}")
 
 
+@pytest.mark.parametrize("s_k", [31, 32, 33, 47, 63, 64, 65, 95, 97, 255, 257, 1055, 1100, 1793, 2047])
+def test_last_key_tile_ends_at_the_last_key(s_k):
+    """The fused kernel fetches 32-key tiles; a tile that would reach past the last key is moved back
+    to end there and the columns that repeat the tile before it must count for nothing.  Sizes on
+    both sides of tile boundaries (31 keys: no whole tile, two-pass path), dense and (B, S, H, D)
+    storage, fp16 (pre-scaled variants for the larger ones: H * rows >= 4096) and bf16, with a
+    strong key in the last real column so that a wrong column mapping shows."""
+    g = torch.Generator().manual_seed(1000 + s_k)
+    b, h = (2, 8) if s_k >= 512 else (3, 4)
+    tq = torch.randn((b, s_k, h, 64), generator=g).half()
+    tk = torch.randn((b, s_k, h, 64), generator=g).half()
+    tk[:, -1] *= 1.5
+    for bf16 in (False, True):
+        q_bshd = (tq.bfloat16() if bf16 else tq).cuda().permute(0, 2, 1, 3)
+        k_bshd = (tk.bfloat16() if bf16 else tk).cuda().permute(0, 2, 1, 3)
+        ref = _oracle(q_bshd.float(), k_bshd.float())
+        out_strided = _run(q_bshd, k_bshd)
+        out_dense = _run(q_bshd.contiguous(), k_bshd.contiguous())
+        _assert_close(out_strided, ref, f"S_k {s_k} bf16 {bf16} (B,S,H,D) storage")
+        _assert_close(out_dense, ref, f"S_k {s_k} bf16 {bf16} dense")
+        assert torch.equal(out_strided, out_dense), f"S_k {s_k} bf16 {bf16}: layouts differ in bits"
+
+
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("scale", [3.0, 2.0])
 def test_key_splits_of_mixed_kind_merge_without_underflow(scale, bf16):
