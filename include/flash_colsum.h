@@ -30,7 +30,7 @@ enum {
     FCS_OK = 0,
     FCS_E_NULL = -1,      /* a required pointer is NULL                                  */
     FCS_E_DIMS = -2,      /* a dimension is < 1, or cls_n == 0, or k_past < 0, or B*H > 65535
-                             on the two-pass path (causal, S > 2048 or D = 128)          */
+                             on the two-pass path (causal, S > 2048, S < 32 or D != 64)   */
     FCS_E_HEAD_DIM = -3,  /* D is not a multiple of 8 in [8, 256]                        */
     FCS_E_STRIDE = -4,    /* last-dim stride != 1, or a stride / base not 16-B aligned   */
     FCS_E_WORKSPACE = -5, /* ws_bytes smaller than fcs_workspace_bytes() for these dims,
