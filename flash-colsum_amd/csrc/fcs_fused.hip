@@ -1,5 +1,5 @@
 // Attention column means on gfx950 (MI355X): fused single-kernel path for non-causal
-// calls whose whole key range fits in one workgroup's registers (S_k <= 2048, D = 64).
+// calls whose whole key range fits in one workgroup's registers (32 <= S_k <= 2048, D = 64).
 //
 // One workgroup = 8 waves.  The waves form a (query group) x (key group) grid; a wave
 // computes the 32 x (32 * tiles) block of scores  S = Q_tile * K_tile^T  for its 32 query
@@ -7,8 +7,8 @@
 // accumulator tiles = 128 VGPRs), so the scores are computed once and exponentiated
 // once.  In this orientation a lane owns one key (column l % 32) and 16 query rows, so the
 // column sums  sum_i e_ij / L_i  are in-lane FMAs; only the row sums L_i cross lanes and
-// waves, once per (head, row block): lanes are folded by a wave-private transpose through
-// LDS, the key-group waves by one workgroup barrier.
+// waves, once per (head, row block): lanes are folded in registers (DPP and lane-swap
+// butterfly), the key-group waves through LDS and one workgroup barrier.
 //
 // Q and K never pass through staging registers: every wave streams its own operands
 // with global_load_lds_dwordx4 into a private LDS ring, several tiles ahead of use, and
@@ -187,9 +187,11 @@ __device__ __forceinline__ floatx4 row_values(const RowRed &rr, int i4, int g)
 // RAGGED = false: S_k is exactly (key groups) x TPW x 32, S_q a multiple of the block's rows and
 //                 the rows of Q and K are dense (row stride == D): every operand tile is whole,
 //                 no padding keys anywhere, and tile addresses need no per-lane arithmetic.
-// RAGGED = true : anything else; fetches compute and clamp their rows per lane and every exponent
-//                 is masked per lane.
-// PRE = 8 or 4 (0 = off; only with RAGGED = false and that many key groups, i.e. 1 or 2 query
+// RAGGED = true : anything else (any 32 <= S_k <= 2048, any S_q, any 16-byte aligned row pitch).  Key
+//                 tiles still need no per-lane arithmetic and no branch: a tile that would reach
+//                 past the last key is moved back to end there, and the columns that then repeat
+//                 the tile before it are given no weight.  Q rows are clamped per lane, once per unit.
+// PRE = 8 or 4 (0 = off; only with that many key groups, i.e. 1 or 2 query
 //                 groups): each query group's Q tile is multiplied by
 //                 c = scale * log2(e) in fp32 ONCE per head, rounded back to fp16 and shared by the
 //                 eight waves through LDS, so the scores leave the MFMAs already in the exponent's
