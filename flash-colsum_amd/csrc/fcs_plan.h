@@ -158,7 +158,16 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     // ---- few-rows path: a batch of matrix-vector products, one workgroup per (batch entry, head group)
     p.fewrows = 0;
     p.fused = 0;
-    if (!causal && p.q_rows <= kFewRowsMaxRows && (long)p.q_rows * Sk <= kFewRowsMaxScores && (D == 64 || D == 128)) {
+    // (One workgroup streams a whole key head and computes its R x Sk scores on the VALU.  The fused
+    // path, which splits a head's keys over eight waves and uses the matrix pipe, is quicker when
+    // there are fewer (batch entry, head) pairs than compute units and a thousand keys or more per
+    // head (B 8, H 16, S 2048, 4 rows: 24 -> 15 us), and when a head has more than 4096 scores
+    // (B 16, H 16, S 2048, 4 rows: 24.4 -> 19.9 us).  The CLS-token shape B 32, H 16, S 577, 1 row
+    // stays here: 13.4 us of kernels against 15.8 us on the fused path.)
+    const bool fused_is_quicker = D == 64 && Sk <= kFusedMaxKeys &&
+                                  ((Sk >= 1024 && (long)B * H < kComputeUnits) || (long)p.q_rows * Sk > 4096);
+    if (!causal && p.q_rows <= kFewRowsMaxRows && (long)p.q_rows * Sk <= kFewRowsMaxScores && (D == 64 || D == 128) &&
+        !fused_is_quicker) {
         p.fewrows = 1;
         const long bh = (long)B * H;
         int hpb = (int)((bh + 2047) / 2048);  // heads per workgroup: about 2048 workgroups at most
