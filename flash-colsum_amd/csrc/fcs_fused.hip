@@ -28,6 +28,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "fcs_device.h"
 #include "fcs_kernels.h"
 
@@ -210,6 +212,17 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // key tile k of every unit sits in slot k % 4 and three key tiles are in flight ahead of the one
     // being used instead of two.
     constexpr bool KRING = PRE && TPW % 4 == 0;
+    // KEEP (KRING with eight tiles per wave): the row blocks of a head, which a workgroup walks one
+    // after the other, use the same key tiles, and the four slots hold half of them.  A unit
+    // therefore leaves its last four key tiles in the ring and the next unit of the same key head
+    // starts with those: units alternate between the tile orders 0..7 and 4..7,0..3 (tile k always
+    // sits in slot k % 4, so every slot number stays a compile-time value), and a unit fetches four
+    // key tiles instead of eight.  Only the first unit of a key head fetches all eight.
+#ifdef FCS_NO_KEEP
+    constexpr bool KEEP = false;
+#else
+    constexpr bool KEEP = KRING && TPW == 8 && !RAGGED;
+#endif
     constexpr int NS = KRING ? 4 : 3;      // ring slots per wave
     constexpr int ITEMS = TPW + 1;         // per (head, row block): the Q tile, then TPW key tiles
     constexpr int SLOT_BYTES = NT * 1024;  // one item: NT pieces x 64 lanes x 16 bytes
@@ -361,8 +374,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     };
 
     float col_acc[TPW];
+    float col_rot[KEEP ? TPW : 1];  // KEEP: sums of the units that ran in the order 4..7,0..3: col_rot[t] belongs to tile t ^ 4
 #pragma unroll
     for (int t = 0; t < TPW; ++t) col_acc[t] = 0.f;
+#pragma unroll
+    for (int t = 0; t < (KEEP ? TPW : 1); ++t) col_rot[t] = 0.f;
+    int rot4 = 0;  // KEEP: 4 while the current unit runs in the order 4..7,0..3
 
     // The walk.  Every head contributes ITEMS = 1 + TPW operand tiles ("items"): its Q tile, then
     // the wave's key tiles.  Item number p (counted over the whole walk) lives in ring slot p % 3.
@@ -469,10 +486,10 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // PRE: scale this wave's raw rows by c (sign included) in fp32, round to fp16 and store them at
     // their swizzled place in the query group's tile of qshare[buf]; a workgroup barrier must
     // follow before they are read
-    auto q_publish = [&](int buf) {
-        // the raw rows were requested one item before the two most recent fetches (2 * NT DMA
-        // instructions): once at most those are outstanding, the rows have landed
-        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(qraw) : "n"(2 * NT) : "memory");
+    auto q_publish = [&](int buf, auto behind_c) {
+        // the raw rows have landed once at most the DMA instructions requested behind them are
+        // outstanding (a compile-time count)
+        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(qraw) : "n"(decltype(behind_c)::value) : "memory");
         const float cs = a.negate ? -a.c : a.c;
         typedef _Float16 qhalf_t __attribute__((ext_vector_type(PRE == 8 ? 4 : 8)));
         const qhalf_t raw = __builtin_bit_cast(qhalf_t, qraw);
@@ -504,7 +521,17 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // step at which the next unit's Q rows are requested (KRING)
     auto ktile_item = [&](int r) { return r < TPW ? 1 + r : ITEMS + 1 + (r - TPW); };
     constexpr int TQ = TPW - 2;
-    if (KRING) {
+    // KEEP: key tile `tile` (wave-uniform, 0..7) of unit `ua` (0 current, 1 next) into ring slot `slot`
+    auto fetch_key_tile = [&](int ua, int tile, int slot) {
+        const char *src = k_b + k_off[ua] + (size_t)((uint32_t)(tile * 32) * k_row_b);
+#pragma unroll
+        for (int tt = 0; tt < NT; ++tt) fetch_piece(src, k_voff, slot, tt);
+    };
+    if (KEEP) {
+        fetch_pos(0, 0);  // the Q rows
+#pragma unroll
+        for (int r = 0; r < NS; ++r) fetch_key_tile(0, r, r);
+    } else if (KRING) {
         // same order of requests as at the end of every unit: key tiles 0 .. NS-3, the Q rows, key tiles
         // NS-2 and NS-1, so that the counted waits below hold for the first unit too
 #pragma unroll
@@ -517,7 +544,8 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         for (int i = 0; i < NS; ++i) fetch_pos(i, i);
     }
     if (PRE) {
-        q_publish(0);
+        // behind the Q rows: KEEP the first four key tiles, else two key tiles
+        q_publish(0, std::integral_constant<int, (KEEP ? NS : 2) * NT>{});
         __syncthreads();
     }
 
@@ -535,7 +563,16 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             FCS_WAIT_VM(2 * NT);
             take_issue(slot_of(0), qf);
         }
-        if (KRING) {
+        // KEEP: does the next unit read another key head (then its first four tiles are fetched during
+        // this unit's last four steps; else they are the ones this unit leaves behind)
+        const bool next_key_head = KEEP && k_off[1] != k_off[0];
+        if (KEEP) {
+            // the unit's first four tiles are in the ring: left by the previous unit, or requested
+            // during its last steps (first unit of a key head), or by the prologue.  Nothing else is
+            // outstanding here, so the common case does not wait.
+            FCS_WAIT_VM(0);
+            take_issue(0, kf[0]);
+        } else if (KRING) {
             // key tile 0 was requested NS steps ago; behind it: NS - 1 key tiles and the Q rows
             FCS_WAIT_VM((NS - 1) * NT + 1);
             take_issue(0, kf[0]);
@@ -580,7 +617,23 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             else asm volatile("s_setprio 0");
             // the operands of this tile were read back during the previous step: they have landed,
             // their ring slots are free again and take the look-ahead fetches
-            if (KRING) {
+            if (KEEP) {
+                if (t == 0) take_wait(qf);
+                take_wait(kf[t & 1]);
+                if (t == TQ) fetch_pos(ITEMS, 0);  // the next unit's Q rows
+                // the slot of this step's tile is free.  Steps 0..3: it takes the tile of step t + 4.
+                // Steps 4..7: nothing, unless the next unit reads another key head: then its tile t - 4.
+                if (t < NS) fetch_key_tile(0, (t + NS) ^ rot4, t);
+                else if (next_key_head) fetch_key_tile(1, t - NS, t - NS);
+                // The tile of step t + 1 (t >= 3) was requested at step t - 3; behind it: the tiles of the
+                // steps up to 3, and the Q rows at step TQ.  (The requests for another key head are not
+                // counted: with them outstanding the waits below only wait for more than they need.)
+                if (t + 1 >= NS && t + 1 < TPW) {
+                    if (t >= TQ) FCS_WAIT_VM(1);
+                    else FCS_WAIT_VM((TPW - 2 - t) * NT);
+                }
+                if (t + 1 < TPW) take_issue((t + 1) % NS, kf[(t + 1) & 1]);
+            } else if (KRING) {
                 if (t == 0) take_wait(qf);
                 take_wait(kf[t & 1]);
                 // the slot of key tile t is free: it takes key tile t + NS; the next unit's Q rows are
@@ -625,14 +678,27 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             sq += ITEMS % NS;
             if (sq >= NS) sq -= NS;
         }
-        if (PRE) q_publish((unit + 1) & 1);  // next head's Q tile; the reduction's barrier publishes it
+        // next unit's Q tile; the reduction's barrier publishes it.  Behind its rows: two key tiles
+        // (KEEP: nothing that may be waited past)
+        if (PRE) q_publish((unit + 1) & 1, std::integral_constant<int, KEEP ? 0 : 2 * NT>{});
 
         // ---------------- row sums over lanes and key-group waves; w = 1/L (0 for rows not averaged)
         const bool slow = reduce_rows<false>(rs, rr, kg_n, qg, kg, lane, [&](int row, float L) {
             return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
         }, PRE ? kSumHiPre : kSumHi);
 
-        if (!slow) {
+        if (!slow && KEEP && rot4) {
+            // ---------------- phase 3 of a unit in the order 4..7,0..3: step t held tile t ^ 4
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const floatx4 w4 = row_values(rr, i4, g);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int t = 0; t < (KEEP ? TPW : 1); ++t) col_rot[t] = fmaf(acc[t][4 * i4 + j], w4[j], col_rot[t]);
+                }
+            }
+        } else if (!slow) {
             // ---------------- phase 3: column sums of e * w
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
@@ -720,6 +786,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                     if (u == t) col_acc[u] += sum;
             }
         }
+        if (KEEP) rot4 = next_key_head ? 0 : (rot4 ^ 4);
         if (++cur_rb == rb_n) {
             cur_rb = 0;
             ++cur_hr;
@@ -732,7 +799,8 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     float *dst = a.partial + ((int64_t)slab * a.B + b) * a.Sk;
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
-        const float v = col_acc[t] + __shfl_xor(col_acc[t], 32);
+        const float both = KEEP ? col_acc[t] + col_rot[(t ^ 4) % (KEEP ? TPW : 1)] : col_acc[t];
+        const float v = both + __shfl_xor(both, 32);
         if (g == 0 && t <= tmax_lane) dst[tile_first(t) + n] = v;
     }
 }
