@@ -221,7 +221,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 #ifdef FCS_NO_KEEP
     constexpr bool KEEP = false;
 #else
-    constexpr bool KEEP = KRING && TPW == 8 && !RAGGED;
+    constexpr bool KEEP = KRING && TPW == 8;
 #endif
     constexpr int NS = KRING ? 4 : 3;      // ring slots per wave
     constexpr int ITEMS = TPW + 1;         // per (head, row block): the Q tile, then TPW key tiles
@@ -523,9 +523,18 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     constexpr int TQ = TPW - 2;
     // KEEP: key tile `tile` (wave-uniform, 0..7) of unit `ua` (0 current, 1 next) into ring slot `slot`
     auto fetch_key_tile = [&](int ua, int tile, int slot) {
-        const char *src = k_b + k_off[ua] + (size_t)((uint32_t)(tile * 32) * k_row_b);
+        if (RAGGED) {
+            const char *src = k_batch + k_off[ua] + (size_t)tile_first(tile) * k_row_b;
 #pragma unroll
-        for (int tt = 0; tt < NT; ++tt) fetch_piece(src, k_voff, slot, tt);
+            for (int tt = 0; tt < NT; ++tt) {
+                FCS_OPAQUE_V(k_voff[tt % NVOFF]);
+                fetch_piece_at(src, k_voff[tt % NVOFF], slot, tt);
+            }
+        } else {
+            const char *src = k_b + k_off[ua] + (size_t)((uint32_t)(tile * 32) * k_row_b);
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) fetch_piece(src, k_voff, slot, tt);
+        }
     };
     if (KEEP) {
         fetch_pos(0, 0);  // the Q rows
@@ -591,7 +600,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             // exponential is 0; the bias rides on the scale multiply (one FMA).  Pre-scaled scores have
             // no multiply to carry it: there the column's exponentials (finite: they repeat real keys)
             // enter the row sums with weight 0 (an FMA in place of the add).
-            const bool counts = !RAGGED || t <= tmax_lane;
+            const bool counts = !RAGGED || (KEEP ? (t ^ rot4) : t) <= tmax_lane;  // KEEP: step t holds tile t ^ rot4
             const float bias = counts ? 0.f : -INFINITY, one = counts ? 1.f : 0.f;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
