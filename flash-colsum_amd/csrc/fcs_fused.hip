@@ -207,26 +207,19 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     static_assert(D == 64, "the fused path is laid out for 64-wide heads");
     static_assert(!(PRE && BF), "the pre-scaled variant rounds Q*c to fp16; bf16 would be too coarse");
     constexpr int NT = D / 16;             // MFMA steps (and 16-byte pieces per lane) per operand tile
-    // KRING (pre-scaled variants whose tile count is a multiple of four): the ring holds key
-    // tiles only, in four slots.  The Q item of those variants is a plain load that needs no slot, so
-    // key tile k of every unit sits in slot k % 4 and three key tiles are in flight ahead of the one
-    // being used instead of two.
-    constexpr bool KRING = PRE && TPW % 4 == 0;
-    // KEEP (KRING with eight tiles per wave): the row blocks of a head, which a workgroup walks one
-    // after the other, use the same key tiles, and the four slots hold half of them.  A unit
-    // therefore leaves its last four key tiles in the ring and the next unit of the same key head
-    // starts with those: units alternate between the tile orders 0..7 and 4..7,0..3 (tile k always
-    // sits in slot k % 4, so every slot number stays a compile-time value), and a unit fetches four
-    // key tiles instead of eight.  Only the first unit of a key head fetches all eight.
-#ifdef FCS_NO_KEEP
-    constexpr bool KEEP = false;
-#else
-    constexpr bool KEEP = KRING && TPW == 8;
-#endif
-    constexpr int NS = KRING ? 4 : 3;      // ring slots per wave
+    // KEEP (pre-scaled variants with eight or six key tiles per wave): the Q item of those variants
+    // is a plain load that needs no ring slot, so the ring holds key tiles only, in NS = TPW / 2
+    // slots, tile k of every unit in slot k % NS (every slot number stays a compile-time value).
+    // The row blocks of a head, which a workgroup walks one after the other, use the same key
+    // tiles: a unit leaves its last NS key tiles in the ring and the next unit of the same key head
+    // starts with those.  Units alternate between the tile orders 0 .. TPW-1 and
+    // NS .. TPW-1, 0 .. NS-1 and fetch NS key tiles each instead of TPW; only the first unit of a
+    // key head fetches all of them.
+    constexpr bool KEEP = PRE && (TPW == 8 || TPW == 6);
+    constexpr int NS = KEEP ? TPW / 2 : 3;  // ring slots per wave
     constexpr int ITEMS = TPW + 1;         // per (head, row block): the Q tile, then TPW key tiles
     constexpr int SLOT_BYTES = NT * 1024;  // one item: NT pieces x 64 lanes x 16 bytes
-    constexpr bool STATIC_SLOTS = KRING || (ITEMS % NS == 0);  // then an item's slot is a compile-time value
+    constexpr bool STATIC_SLOTS = KEEP || (ITEMS % NS == 0);  // then an item's slot is a compile-time value
     __shared__ __attribute__((aligned(16))) char ring[8 * NS * SLOT_BYTES];
     __shared__ __attribute__((aligned(16))) float part[2 * 256];
     __shared__ __attribute__((aligned(16))) float wv[8 * 32];
@@ -374,12 +367,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     };
 
     float col_acc[TPW];
-    float col_rot[KEEP ? TPW : 1];  // KEEP: sums of the units that ran in the order 4..7,0..3: col_rot[t] belongs to tile t ^ 4
+    float col_rot[KEEP ? TPW : 1];  // KEEP: sums of the units that ran in the rotated order: col_rot[t] belongs to tile (t + NS) % TPW
 #pragma unroll
     for (int t = 0; t < TPW; ++t) col_acc[t] = 0.f;
 #pragma unroll
     for (int t = 0; t < (KEEP ? TPW : 1); ++t) col_rot[t] = 0.f;
-    int rot4 = 0;  // KEEP: 4 while the current unit runs in the order 4..7,0..3
+    int rot = 0;  // KEEP: 1 while the current unit runs in the rotated order NS .. TPW-1, 0 .. NS-1
 
     // The walk.  Every head contributes ITEMS = 1 + TPW operand tiles ("items"): its Q tile, then
     // the wave's key tiles.  Item number p (counted over the whole walk) lives in ring slot p % 3.
@@ -391,9 +384,9 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     //     instructions at every wait is a compile-time constant.
     // PRE: the Q item of a head is not a tile in the ring but this wave's 32 / PRE rows of its query
     // group's raw tile (512 B or 1 KB), one ordinary 8- or 16-byte load per lane; the wave scales
-    // them and publishes them in `qshare`.  KRING: that item then takes no slot number either; key
-    // tile k of every unit lives in slot k % 4, key tile k + 4 is fetched when tile k has been read
-    // back, and the next unit's Q rows are requested at step TPW - 2.
+    // them and publishes them in `qshare`.  KEEP: that item then takes no slot number either; key
+    // tile k of every unit lives in slot k % NS, a unit requests the second half of its tile order
+    // while it reads back the first, and the next unit's Q rows at step TPW - 2.
     // raw Q rows of the pre-scaled variant: written by an asynchronous load and read after a hand-placed
     // wait, so the variable the load names must be the one the wait names (no copies in between)
     typedef uint32_t qraw_t __attribute__((ext_vector_type(PRE == 8 ? 2 : 4)));
@@ -517,11 +510,8 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     };
 
     half8 qf[NT], kf[2][NT];
-    // item of key tile r counted from the current unit's first (r >= TPW: the next unit's), and the
-    // step at which the next unit's Q rows are requested (KRING)
-    auto ktile_item = [&](int r) { return r < TPW ? 1 + r : ITEMS + 1 + (r - TPW); };
-    constexpr int TQ = TPW - 2;
-    // KEEP: key tile `tile` (wave-uniform, 0..7) of unit `ua` (0 current, 1 next) into ring slot `slot`
+    constexpr int TQ = TPW - 2;  // KEEP: the step at which the next unit's Q rows are requested
+    // KEEP: key tile `tile` (wave-uniform, 0 .. TPW-1) of unit `ua` (0 current, 1 next) into ring slot `slot`
     auto fetch_key_tile = [&](int ua, int tile, int slot) {
         if (RAGGED) {
             const char *src = k_batch + k_off[ua] + (size_t)tile_first(tile) * k_row_b;
@@ -540,20 +530,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         fetch_pos(0, 0);  // the Q rows
 #pragma unroll
         for (int r = 0; r < NS; ++r) fetch_key_tile(0, r, r);
-    } else if (KRING) {
-        // same order of requests as at the end of every unit: key tiles 0 .. NS-3, the Q rows, key tiles
-        // NS-2 and NS-1, so that the counted waits below hold for the first unit too
-#pragma unroll
-        for (int r = 0; r < NS - 2; ++r) fetch_pos(ktile_item(r), r);
-        fetch_pos(0, 0);
-        fetch_pos(ktile_item(NS - 2), NS - 2);
-        fetch_pos(ktile_item(NS - 1), NS - 1);
     } else {
 #pragma unroll
         for (int i = 0; i < NS; ++i) fetch_pos(i, i);
     }
     if (PRE) {
-        // behind the Q rows: KEEP the first four key tiles, else two key tiles
+        // behind the Q rows: KEEP the first NS key tiles, else two key tiles
         q_publish(0, std::integral_constant<int, (KEEP ? NS : 2) * NT>{});
         __syncthreads();
     }
@@ -572,18 +554,14 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             FCS_WAIT_VM(2 * NT);
             take_issue(slot_of(0), qf);
         }
-        // KEEP: does the next unit read another key head (then its first four tiles are fetched during
-        // this unit's last four steps; else they are the ones this unit leaves behind)
+        // KEEP: does the next unit read another key head (then its first NS tiles are fetched during
+        // this unit's last NS steps; else they are the ones this unit leaves behind)
         const bool next_key_head = KEEP && k_off[1] != k_off[0];
         if (KEEP) {
-            // the unit's first four tiles are in the ring: left by the previous unit, or requested
+            // the unit's first NS tiles are in the ring: left by the previous unit, or requested
             // during its last steps (first unit of a key head), or by the prologue.  Nothing else is
             // outstanding here, so the common case does not wait.
             FCS_WAIT_VM(0);
-            take_issue(0, kf[0]);
-        } else if (KRING) {
-            // key tile 0 was requested NS steps ago; behind it: NS - 1 key tiles and the Q rows
-            FCS_WAIT_VM((NS - 1) * NT + 1);
             take_issue(0, kf[0]);
         } else {
             FCS_WAIT_VM(1 * NT);
@@ -600,7 +578,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             // exponential is 0; the bias rides on the scale multiply (one FMA).  Pre-scaled scores have
             // no multiply to carry it: there the column's exponentials (finite: they repeat real keys)
             // enter the row sums with weight 0 (an FMA in place of the add).
-            const bool counts = !RAGGED || (KEEP ? (t ^ rot4) : t) <= tmax_lane;  // KEEP: step t holds tile t ^ rot4
+            const bool counts = !RAGGED || ((KEEP && rot) ? (t + NS) % TPW : t) <= tmax_lane;  // a rotated unit's step t holds tile (t + NS) % TPW
             const float bias = counts ? 0.f : -INFINITY, one = counts ? 1.f : 0.f;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -630,31 +608,17 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 if (t == 0) take_wait(qf);
                 take_wait(kf[t & 1]);
                 if (t == TQ) fetch_pos(ITEMS, 0);  // the next unit's Q rows
-                // the slot of this step's tile is free.  Steps 0..3: it takes the tile of step t + 4.
-                // Steps 4..7: nothing, unless the next unit reads another key head: then its tile t - 4.
-                if (t < NS) fetch_key_tile(0, (t + NS) ^ rot4, t);
+                // the slot of this step's tile is free.  First NS steps: it takes the tile of step t + NS.
+                // Last NS steps: nothing, unless the next unit reads another key head: then its tile t - NS.
+                if (t < NS) fetch_key_tile(0, rot ? t : t + NS, t);
                 else if (next_key_head) fetch_key_tile(1, t - NS, t - NS);
-                // The tile of step t + 1 (t >= 3) was requested at step t - 3; behind it: the tiles of the
-                // steps up to 3, and the Q rows at step TQ.  (The requests for another key head are not
+                // The tile of step t + 1 (t + 1 >= NS) was requested at step t + 1 - NS; behind it: the tiles
+                // requested at the steps up to NS - 1, and the Q rows at step TQ.  (The requests for another key head are not
                 // counted: with them outstanding the waits below only wait for more than they need.)
                 if (t + 1 >= NS && t + 1 < TPW) {
                     if (t >= TQ) FCS_WAIT_VM(1);
                     else FCS_WAIT_VM((TPW - 2 - t) * NT);
                 }
-                if (t + 1 < TPW) take_issue((t + 1) % NS, kf[(t + 1) & 1]);
-            } else if (KRING) {
-                if (t == 0) take_wait(qf);
-                take_wait(kf[t & 1]);
-                // the slot of key tile t is free: it takes key tile t + NS; the next unit's Q rows are
-                // requested at step TQ, before that step's key tile
-                if (t == TQ) fetch_pos(ITEMS, 0);
-                fetch_pos(ktile_item(t + NS), t % NS);
-                // key tile t + 1 has landed once only what was requested behind it is outstanding: the
-                // NS - 1 key tiles of steps t + 2 - NS .. t, and the Q rows if their step is among those
-                constexpr int TQ_PREV = TQ - TPW;  // the previous unit's request, seen from this unit
-                const bool q_behind = (TQ >= t + 2 - NS && TQ <= t) || (TQ_PREV >= t + 2 - NS && TQ_PREV <= t);
-                if (q_behind) FCS_WAIT_VM((NS - 1) * NT + 1);
-                else FCS_WAIT_VM((NS - 1) * NT);
                 if (t + 1 < TPW) take_issue((t + 1) % NS, kf[(t + 1) & 1]);
             } else {
             if (t == 0) {
@@ -696,8 +660,8 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
         }, PRE ? kSumHiPre : kSumHi);
 
-        if (!slow && KEEP && rot4) {
-            // ---------------- phase 3 of a unit in the order 4..7,0..3: step t held tile t ^ 4
+        if (!slow && KEEP && rot) {
+            // ---------------- phase 3 of a unit in the rotated order: step t held tile (t + NS) % TPW
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const floatx4 w4 = row_values(rr, i4, g);
@@ -795,7 +759,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                     if (u == t) col_acc[u] += sum;
             }
         }
-        if (KEEP) rot4 = next_key_head ? 0 : (rot4 ^ 4);
+        if (KEEP) rot = next_key_head ? 0 : (rot ^ 1);
         if (++cur_rb == rb_n) {
             cur_rb = 0;
             ++cur_hr;
@@ -808,7 +772,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     float *dst = a.partial + ((int64_t)slab * a.B + b) * a.Sk;
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
-        const float both = KEEP ? col_acc[t] + col_rot[(t ^ 4) % (KEEP ? TPW : 1)] : col_acc[t];
+        const float both = KEEP ? col_acc[t] + col_rot[KEEP ? (t + NS) % TPW : 0] : col_acc[t];
         const float v = both + __shfl_xor(both, 32);
         if (g == 0 && t <= tmax_lane) dst[tile_first(t) + n] = v;
     }
