@@ -809,6 +809,30 @@ def test_fused_path_with_several_row_blocks_per_workgroup(qs, ks, kw):
     _assert_close(out, ref, f"{qs} {ks} {kw}")
 
 
+@pytest.mark.parametrize("qs,ks,kw", [
+    ((3, 6, 2048, 64), (3, 6, 2048, 64), {}),                       # eight tiles per wave, several heads per workgroup
+    ((1, 5, 2048, 64), (1, 5, 2048, 64), {"cls_len": 1500}),        # an odd number of row blocks per head
+    ((2, 16, 1536, 64), (2, 16, 1536, 64), {}),                     # six tiles per wave, three ring slots
+    ((5, 8, 1370, 64), (5, 8, 1370, 64), {}),                       # six tiles, the last one moved back
+    ((2, 8, 2048, 64), (2, 2, 2048, 64), {}),                       # grouped key heads: four query heads per key head
+    ((2, 12, 1000, 64), (2, 4, 1536, 64), {}),                      # grouped, S_q != S_k
+    ((4, 4, 1024, 64), (4, 4, 1024, 64), {"scale": -0.125}),        # two query groups per workgroup, negated scores
+])
+def test_key_tiles_kept_between_row_blocks(qs, ks, kw):
+    """The pre-scaled fused variants with eight or six key tiles per wave leave half of a head's key
+    tiles in the LDS ring for the next row block of the same key head and walk the tiles in two
+    alternating orders.  Distinct keys per tile and per head, so that a tile read from the wrong
+    slot, a stale tile after a change of key head, or column sums added to the wrong tile show."""
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn(qs, generator=g).half()
+    k = torch.randn(ks, generator=g).half()
+    k *= (1.0 + 0.25 * torch.arange(ks[1]).view(1, -1, 1, 1) / ks[1]).half()   # heads differ in scale
+    k[:, :, ::97] *= 1.5                                                       # a few strong keys spread over the tiles
+    out, ref = _run_ext(q, k, **kw), _oracle_ext(q.float().cuda(), k.float().cuda(), **kw)
+    _assert_close(out, ref, f"{qs} {ks} {kw}")
+    assert torch.equal(out, _run_ext(q, k, **kw)), "not reproducible"
+
+
 @pytest.mark.parametrize("s_k", [31, 32, 33, 47, 63, 64, 65, 95, 97, 255, 257, 1055, 1100, 1793, 2047])
 def test_last_key_tile_ends_at_the_last_key(s_k):
     """The fused kernel fetches 32-key tiles; a tile that would reach past the last key is moved back
