@@ -193,6 +193,10 @@ __device__ __forceinline__ floatx4 row_values(const RowRed &rr, int i4, int g)
 //                 tiles still need no per-lane arithmetic and no branch: a tile that would reach
 //                 past the last key is moved back to end there, and the columns that then repeat
 //                 the tile before it are given no weight.  Q rows are clamped per lane, once per unit.
+// QS (only with PRE): true = the shared Q tile is pre-scaled as described next; false = it is shared
+//                 as it is (any operand type, any scale, any number of averaged rows; the sign of a
+//                 negative scale is applied to it) and every score is still multiplied by c: the
+//                 variant exists for the key-only ring, see KEEP below.
 // PRE = 8 or 4 (0 = off; only with that many key groups, i.e. 1 or 2 query
 //                 groups): each query group's Q tile is multiplied by
 //                 c = scale * log2(e) in fp32 ONCE per head, rounded back to fp16 and shared by the
@@ -201,11 +205,12 @@ __device__ __forceinline__ floatx4 row_values(const RowRed &rr, int i4, int g)
 //                 each score by ~2^-12 relative; the launcher only picks this variant when at least
 //                 4096 (head, row) pairs are averaged per output, where the effect on the means is
 //                 below 1e-4 relative (measured 6.5e-5 at B8 H16 S2048).
-template <int D, int TPW, bool RAGGED, int PRE, bool BF>
+template <int D, int TPW, bool RAGGED, int PRE, bool BF, bool QS = true>
 __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 {
     static_assert(D == 64, "the fused path is laid out for 64-wide heads");
-    static_assert(!(PRE && BF), "the pre-scaled variant rounds Q*c to fp16; bf16 would be too coarse");
+    static_assert(!(PRE && QS && BF), "the pre-scaled variant rounds Q*c to fp16; bf16 would be too coarse");
+    constexpr bool PRESCALED = PRE && QS;  // scores leave the MFMAs in the exponent's unit
     constexpr int NT = D / 16;             // MFMA steps (and 16-byte pieces per lane) per operand tile
     // KEEP (pre-scaled variants with eight or six key tiles per wave): the Q item of those variants
     // is a plain load that needs no ring slot, so the ring holds key tiles only, in NS = TPW / 2
@@ -483,12 +488,21 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         // the raw rows have landed once at most the DMA instructions requested behind them are
         // outstanding (a compile-time count)
         asm volatile("s_waitcnt vmcnt(%1)" : "+v"(qraw) : "n"(decltype(behind_c)::value) : "memory");
-        const float cs = a.negate ? -a.c : a.c;
-        typedef _Float16 qhalf_t __attribute__((ext_vector_type(PRE == 8 ? 4 : 8)));
-        const qhalf_t raw = __builtin_bit_cast(qhalf_t, qraw);
         half8 sc = kZero8;
+        if (QS) {
+            const float cs = a.negate ? -a.c : a.c;
+            typedef _Float16 qhalf_t __attribute__((ext_vector_type(PRE == 8 ? 4 : 8)));
+            const qhalf_t raw = __builtin_bit_cast(qhalf_t, qraw);
 #pragma unroll
-        for (int e = 0; e < (PRE == 8 ? 4 : 8); ++e) sc[e] = (_Float16)((float)raw[e] * cs);
+            for (int e = 0; e < (PRE == 8 ? 4 : 8); ++e) sc[e] = (_Float16)((float)raw[e] * cs);
+        } else {
+            // shared as it is: only the sign bit of every 16-bit value (fp16 and bf16 alike) follows the scale's sign
+            uint4v u = {0u, 0u, 0u, 0u};
+            const uint32_t flip = a.negate ? 0x80008000u : 0u;
+#pragma unroll
+            for (int e = 0; e < (PRE == 8 ? 2 : 4); ++e) u[e] = qraw[e] ^ flip;
+            sc = __builtin_bit_cast(half8, u);
+        }
         char *tile = qshare + (buf * PQG + qg) * 4096;
         if (PRE == 8) {  // 4 rows per wave, 8 bytes per lane
             const int row = kg * 4 + (lane >> 4), pc = (lane & 15) >> 1, hf = lane & 1;
@@ -582,9 +596,9 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             const float bias = counts ? 0.f : -INFINITY, one = counts ? 1.f : 0.f;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const float e = fast_exp2(PRE ? acc[t][i] : (RAGGED ? fmaf(acc[t][i], a.c, bias) : acc[t][i] * a.c));
+                const float e = fast_exp2(PRESCALED ? acc[t][i] : (RAGGED ? fmaf(acc[t][i], a.c, bias) : acc[t][i] * a.c));
                 acc[t][i] = e;
-                if (PRE && RAGGED) rs[i] = fmaf(e, one, rs[i]);
+                if (PRESCALED && RAGGED) rs[i] = fmaf(e, one, rs[i]);
                 else rs[i] += e;
             }
             // pinned here: otherwise the optimiser sinks every exponent below the last MFMA
@@ -658,7 +672,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         // ---------------- row sums over lanes and key-group waves; w = 1/L (0 for rows not averaged)
         const bool slow = reduce_rows<false>(rs, rr, kg_n, qg, kg, lane, [&](int row, float L) {
             return (blk_row0 + row < a.q_rows) ? __builtin_amdgcn_rcpf(L) : 0.f;
-        }, PRE ? kSumHiPre : kSumHi);
+        }, PRESCALED ? kSumHiPre : kSumHi);
 
         if (!slow && KEEP && rot) {
             // ---------------- phase 3 of a unit in the rotated order: step t held tile (t + NS) % TPW
@@ -785,6 +799,17 @@ static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
     const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
     const bool pre = !BF && TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4) && (long)p.H * p.q_rows >= 4096 &&
                      fabsf(a.c) <= 0.1251f * 1.44269504f;
+    // the other calls with eight or six tiles per wave: Q shared through LDS as it is, key-only ring
+    constexpr int TPWS = (TPW == 6) ? 6 : 8;
+    const bool shared_q = !pre && (TPW == 8 || TPW == 6) && (p.f_kg == 8 || p.f_kg == 4);
+    if (shared_q && p.f_kg == 8) {
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 8, BF, false>), grid, dim3(512), 0, st, a);
+        return;
+    }
+    if (shared_q) {
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 4, BF, false>), grid, dim3(512), 0, st, a);
+        return;
+    }
     if (pre && whole && TPW == 8 && p.f_kg == 8)
         hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 8, false>), grid, dim3(512), 0, st, a);
     else if (pre && whole && TPW == 8 && p.f_kg == 4)
