@@ -212,19 +212,24 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     static_assert(!(PRE && QS && BF), "the pre-scaled variant rounds Q*c to fp16; bf16 would be too coarse");
     constexpr bool PRESCALED = PRE && QS;  // scores leave the MFMAs in the exponent's unit
     constexpr int NT = D / 16;             // MFMA steps (and 16-byte pieces per lane) per operand tile
-    // KEEP (pre-scaled variants with eight or six key tiles per wave): the Q item of those variants
-    // is a plain load that needs no ring slot, so the ring holds key tiles only, in NS = TPW / 2
-    // slots, tile k of every unit in slot k % NS (every slot number stays a compile-time value).
-    // The row blocks of a head, which a workgroup walks one after the other, use the same key
-    // tiles: a unit leaves its last NS key tiles in the ring and the next unit of the same key head
-    // starts with those.  Units alternate between the tile orders 0 .. TPW-1 and
-    // NS .. TPW-1, 0 .. NS-1 and fetch NS key tiles each instead of TPW; only the first unit of a
-    // key head fetches all of them.
-    constexpr bool KEEP = PRE && (TPW == 8 || TPW == 6);
-    constexpr int NS = KEEP ? TPW / 2 : 3;  // ring slots per wave
+    // KEEP (shared-Q variants with five to eight key tiles per wave): the Q item of those variants is
+    // a plain load that needs no ring slot, so the ring holds key tiles only, tile k of every unit in
+    // slot k % NS.  The row blocks of a head, which a workgroup walks one after the other, use the
+    // same key tiles: a unit leaves its last NS key tiles in the ring and the next unit of the same
+    // key head starts with those, walking the tiles in another order, and fetches TPW - NS key tiles
+    // instead of TPW; only the first unit of a key head fetches all of them.  Two orders alternate:
+    //   * eight or six tiles (NS = TPW / 2): 0 .. TPW-1 and NS .. TPW-1, 0 .. NS-1; step t then
+    //     always uses slot t % NS, a compile-time value;
+    //   * seven or five tiles (NS = 4): 0 .. TPW-1 and TPW-1 .. 0; the slot of a step depends on
+    //     the order and is added to the read-back addresses at run time.
+    // Each order has its own column sums; they are added at the end.
+    constexpr bool KEEP_ROT = PRE && (TPW == 8 || TPW == 6);
+    constexpr bool KEEP_REV = PRE && (TPW == 7 || TPW == 5);
+    constexpr bool KEEP = KEEP_ROT || KEEP_REV;
+    constexpr int NS = KEEP_ROT ? TPW / 2 : KEEP_REV ? 4 : 3;  // ring slots per wave
     constexpr int ITEMS = TPW + 1;         // per (head, row block): the Q tile, then TPW key tiles
     constexpr int SLOT_BYTES = NT * 1024;  // one item: NT pieces x 64 lanes x 16 bytes
-    constexpr bool STATIC_SLOTS = KEEP || (ITEMS % NS == 0);  // then an item's slot is a compile-time value
+    constexpr bool STATIC_SLOTS = KEEP_ROT || (!KEEP_REV && ITEMS % NS == 0);  // then an item's slot is a compile-time value
     __shared__ __attribute__((aligned(16))) char ring[8 * NS * SLOT_BYTES];
     __shared__ __attribute__((aligned(16))) float part[2 * 256];
     __shared__ __attribute__((aligned(16))) float wv[8 * 32];
@@ -372,12 +377,15 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     };
 
     float col_acc[TPW];
-    float col_rot[KEEP ? TPW : 1];  // KEEP: sums of the units that ran in the rotated order: col_rot[t] belongs to tile (t + NS) % TPW
+    float col_rot[KEEP ? TPW : 1];  // KEEP: sums of the units that ran in the second order: col_rot[t] belongs to tile tile_of(t)
 #pragma unroll
     for (int t = 0; t < TPW; ++t) col_acc[t] = 0.f;
 #pragma unroll
     for (int t = 0; t < (KEEP ? TPW : 1); ++t) col_rot[t] = 0.f;
-    int rot = 0;  // KEEP: 1 while the current unit runs in the rotated order NS .. TPW-1, 0 .. NS-1
+    int rot = 0;  // KEEP: 1 while the current unit runs in the second order
+    // KEEP: the key tile of step t (compile-time) of the current unit, and its ring slot
+    auto tile_of = [&](int t) { return !rot ? t : KEEP_ROT ? (t + NS) % TPW : TPW - 1 - t; };
+    auto slot_of_step = [&](int t) { return KEEP_ROT ? t % NS : tile_of(t) % NS; };
 
     // The walk.  Every head contributes ITEMS = 1 + TPW operand tiles ("items"): its Q tile, then
     // the wave's key tiles.  Item number p (counted over the whole walk) lives in ring slot p % 3.
@@ -569,14 +577,14 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             take_issue(slot_of(0), qf);
         }
         // KEEP: does the next unit read another key head (then its first NS tiles are fetched during
-        // this unit's last NS steps; else they are the ones this unit leaves behind)
+        // this unit's last NS steps, in the first order; else they are the ones this unit leaves behind)
         const bool next_key_head = KEEP && k_off[1] != k_off[0];
         if (KEEP) {
             // the unit's first NS tiles are in the ring: left by the previous unit, or requested
             // during its last steps (first unit of a key head), or by the prologue.  Nothing else is
             // outstanding here, so the common case does not wait.
             FCS_WAIT_VM(0);
-            take_issue(0, kf[0]);
+            take_issue(slot_of_step(0), kf[0]);
         } else {
             FCS_WAIT_VM(1 * NT);
             take_issue(slot_of(1), kf[0]);
@@ -592,7 +600,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             // exponential is 0; the bias rides on the scale multiply (one FMA).  Pre-scaled scores have
             // no multiply to carry it: there the column's exponentials (finite: they repeat real keys)
             // enter the row sums with weight 0 (an FMA in place of the add).
-            const bool counts = !RAGGED || ((KEEP && rot) ? (t + NS) % TPW : t) <= tmax_lane;  // a rotated unit's step t holds tile (t + NS) % TPW
+            const bool counts = !RAGGED || (KEEP ? tile_of(t) : t) <= tmax_lane;
             const float bias = counts ? 0.f : -INFINITY, one = counts ? 1.f : 0.f;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -622,18 +630,21 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 if (t == 0) take_wait(qf);
                 take_wait(kf[t & 1]);
                 if (t == TQ) fetch_pos(ITEMS, 0);  // the next unit's Q rows
-                // the slot of this step's tile is free.  First NS steps: it takes the tile of step t + NS.
-                // Last NS steps: nothing, unless the next unit reads another key head: then its tile t - NS.
-                if (t < NS) fetch_key_tile(0, rot ? t : t + NS, t);
-                else if (next_key_head) fetch_key_tile(1, t - NS, t - NS);
-                // The tile of step t + 1 (t + 1 >= NS) was requested at step t + 1 - NS; behind it: the tiles
-                // requested at the steps up to NS - 1, and the Q rows at step TQ.  (The requests for another key head are not
-                // counted: with them outstanding the waits below only wait for more than they need.)
+                // The slot of this step's tile is free.  It takes the tile of step t + NS (which shares the
+                // slot) if the unit has that step; else nothing, unless the next unit reads another key
+                // head: then the tile of that head that belongs in this slot (its first NS tiles, one per
+                // slot, over the unit's last NS steps).
+                if (t + NS < TPW) fetch_key_tile(0, tile_of(t + NS), slot_of_step(t));
+                else if (next_key_head) fetch_key_tile(1, slot_of_step(t), slot_of_step(t));
+                // The tile of step t + 1 (t + 1 >= NS) was requested at step t + 1 - NS; behind it: the
+                // tiles requested at the later steps, up to step TPW - NS - 1, and the Q rows at step TQ.
+                // (The requests for another key head are not counted: with them outstanding the waits
+                // below only wait for more than they need.)
                 if (t + 1 >= NS && t + 1 < TPW) {
                     if (t >= TQ) FCS_WAIT_VM(1);
                     else FCS_WAIT_VM((TPW - 2 - t) * NT);
                 }
-                if (t + 1 < TPW) take_issue((t + 1) % NS, kf[(t + 1) & 1]);
+                if (t + 1 < TPW) take_issue(slot_of_step(t + 1), kf[(t + 1) & 1]);
             } else {
             if (t == 0) {
                 take_wait(qf);
@@ -675,7 +686,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         }, PRESCALED ? kSumHiPre : kSumHi);
 
         if (!slow && KEEP && rot) {
-            // ---------------- phase 3 of a unit in the rotated order: step t held tile (t + NS) % TPW
+            // ---------------- phase 3 of a unit in the second order: step t held tile tile_of(t)
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const floatx4 w4 = row_values(rr, i4, g);
@@ -786,7 +797,8 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     float *dst = a.partial + ((int64_t)slab * a.B + b) * a.Sk;
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
-        const float both = KEEP ? col_acc[t] + col_rot[KEEP ? (t + NS) % TPW : 0] : col_acc[t];
+        // KEEP: tile t was held by step (t + NS) % TPW (rotated order) or TPW - 1 - t (reversed order) of the units in the second order
+        const float both = KEEP ? col_acc[t] + col_rot[KEEP_ROT ? (t + NS) % TPW : KEEP_REV ? TPW - 1 - t : 0] : col_acc[t];
         const float v = both + __shfl_xor(both, 32);
         if (g == 0 && t <= tmax_lane) dst[tile_first(t) + n] = v;
     }
@@ -799,9 +811,9 @@ static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
     const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
     const bool pre = !BF && TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4) && (long)p.H * p.q_rows >= 4096 &&
                      fabsf(a.c) <= 0.1251f * 1.44269504f;
-    // the other calls with eight or six tiles per wave: Q shared through LDS as it is, key-only ring
-    constexpr int TPWS = (TPW == 6) ? 6 : 8;
-    const bool shared_q = !pre && (TPW == 8 || TPW == 6) && (p.f_kg == 8 || p.f_kg == 4);
+    // the other calls with five to eight tiles per wave: Q shared through LDS as it is, key-only ring
+    constexpr int TPWS = (TPW >= 5) ? TPW : 8;
+    const bool shared_q = !pre && TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4);
     if (shared_q && p.f_kg == 8) {
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 8, BF, false>), grid, dim3(512), 0, st, a);
         return;
