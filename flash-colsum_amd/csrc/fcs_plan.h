@@ -211,7 +211,10 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
                 const int hg = ceil_div(H, hpg);
                 if (ceil_div(H, hg) != hpg) continue;  // same grouping as a smaller hpg
                 const long gens = ((long)nwgq * B * hg + kComputeUnits - 1) / kComputeUnits;
-                double cost = (double)gens * ((double)hpg * rbpw + 0.7) + 0.01 * hg + 0.002 * rbpw;
+                // a unit that follows another row block of the same head finds half of its key tiles in
+                // the LDS ring (the shared-Q kernels; measured 4 % of a unit): row blocks per head count
+                // a little less than heads
+                double cost = (double)gens * ((double)hpg * (rbpw - 0.04 * (rbpw - 1)) + 0.7) + 0.01 * hg + 0.002 * rbpw;
                 // The 32 workgroups that an XCD runs at a time are neighbours in launch order: nwgq of
                 // them share a batch entry, i.e. one head's keys.  When the key heads they stream at
                 // the same time outgrow the XCD's 4 MiB L2, the re-reads of a head's keys by its row
