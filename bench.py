@@ -44,13 +44,13 @@ WORKLOADS = {
     "causal_h32_q512_k65536_d128_peaky": ((1, 32, 512, 128), (1, 32, 65536, 128), dict(is_causal=True), False),
 }
 KERNELS_OF = {
-    "noncausal_b2_h4_s512_d64": "fcs_fused_kernel<64,8,false,0,false> + fcs_finalize_kernel (one call)",
-    "noncausal_b8_h16_s2048_d64": "fcs_fused_kernel<64,8,false,8,false> + fcs_finalize_kernel (one call; the fused kernel is >= 96 % of it)",
-    "cls1_b32_h16_s577_d64": "fcs_fewrows_kernel<64,1> + fcs_finalize_kernel (one call)",
-    "noncausal_b256_h16_s1024_d64": "fcs_fused_kernel<64,8,false,4,false> + fcs_finalize_kernel (one call)",
-    "causal_h32_q128_k4096_d128": "fcs_rowstream_kernel<128,1,4> + fcs_colstream_kernel<128,1,4> + fcs_finalize_kernel (one call)",
-    "causal_h32_q128_k16384_d128": "fcs_rowstream_kernel<128,1,4> + fcs_colstream_kernel<128,1,4> + fcs_finalize_kernel (one call)",
-    "causal_h32_q512_k65536_d128_peaky": "fcs_rowstream_kernel<128,2,8> + fcs_colstream_kernel<128,2,8> + fcs_finalize_kernel (one call)",
+    "noncausal_b2_h4_s512_d64": "fcs_fused_kernel<64,8,false,0,false,true> + fcs_finalize_kernel<32> (one call)",
+    "noncausal_b8_h16_s2048_d64": "fcs_fused_kernel<64,8,false,8,false,true> + fcs_finalize_kernel<8> (one call; the fused kernel is >= 96 % of it)",
+    "cls1_b32_h16_s577_d64": "fcs_fewrows_kernel<64,1> + fcs_finalize_kernel<8> (one call)",
+    "noncausal_b256_h16_s1024_d64": "fcs_fused_kernel<64,8,false,4,false,true> + fcs_finalize_kernel<8> (one call)",
+    "causal_h32_q128_k4096_d128": "fcs_rowstream_kernel<128,1,4> + fcs_colstream_kernel<128,1,4> + fcs_finalize_kernel<8> (one call)",
+    "causal_h32_q128_k16384_d128": "fcs_rowstream_kernel<128,1,4> + fcs_colstream_kernel<128,1,4> + fcs_finalize_kernel<8> (one call)",
+    "causal_h32_q512_k65536_d128_peaky": "fcs_rowstream_kernel<128,2,8> + fcs_colstream_kernel<128,2,8> + fcs_finalize_kernel<8> (one call)",
 }
 DEFAULT = "noncausal_b8_h16_s2048_d64"
 SETTLE_CALLS = 150  # untimed, before the --warmup steps
