@@ -220,13 +220,17 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // instead of TPW; only the first unit of a key head fetches all of them.  Two orders alternate:
     //   * eight or six tiles (NS = TPW / 2): 0 .. TPW-1 and NS .. TPW-1, 0 .. NS-1; step t then
     //     always uses slot t % NS, a compile-time value;
-    //   * seven or five tiles (NS = 4): 0 .. TPW-1 and TPW-1 .. 0; the slot of a step depends on
+    //   * otherwise (NS = 4, or 3 with two key groups): 0 .. TPW-1 and TPW-1 .. 0; the slot of a step depends on
     //     the order and is added to the read-back addresses at run time.
     // Each order has its own column sums; they are added at the end.
-    constexpr bool KEEP_ROT = PRE && (TPW == 8 || TPW == 6);
-    constexpr bool KEEP_REV = PRE && (TPW == 7 || TPW == 5);
+    // (With two key groups there are four query groups: their Q tiles take 32 KB and leave room for
+    // three slots per wave, so eight tiles walk ascending / descending too.)
+    constexpr bool KEEP_ROT = PRE && (TPW == 6 || (TPW == 8 && PRE != 2));
+    constexpr bool KEEP_REV = PRE && !KEEP_ROT;
     constexpr bool KEEP = KEEP_ROT || KEEP_REV;
-    constexpr int NS = KEEP_ROT ? TPW / 2 : KEEP_REV ? 4 : 3;  // ring slots per wave
+    constexpr int NS = KEEP_ROT ? TPW / 2 : KEEP_REV ? (PRE == 2 ? 3 : 4) : 3;  // ring slots per wave
+    constexpr int QV = (PRE == 2) ? 2 : 1;  // load instructions of a wave's share of the raw Q rows
+    static_assert(!PRE || (TPW >= 5 && TPW <= 8), "the shared-Q variants are written for five to eight key tiles per wave");
     constexpr int ITEMS = TPW + 1;         // per (head, row block): the Q tile, then TPW key tiles
     constexpr int SLOT_BYTES = NT * 1024;  // one item: NT pieces x 64 lanes x 16 bytes
     constexpr bool STATIC_SLOTS = KEEP_ROT || (!KEEP_REV && ITEMS % NS == 0);  // then an item's slot is a compile-time value
@@ -403,7 +407,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // raw Q rows of the pre-scaled variant: written by an asynchronous load and read after a hand-placed
     // wait, so the variable the load names must be the one the wait names (no copies in between)
     typedef uint32_t qraw_t __attribute__((ext_vector_type(PRE == 8 ? 2 : 4)));
-    qraw_t qraw = {};
+    qraw_t qraw = {}, qraw_hi = {};  // qraw_hi: the second 16 bytes of a lane (two key groups: 32 bytes per lane)
     auto item_vm = [&](int j_ahead) { return (PRE && (j_ahead % ITEMS) == 0) ? 1 : NT; };  // VMEM instructions of an item
     // What the fetches need to know of the current unit and of the units the look-ahead reaches,
     // refreshed once per unit instead of at every fetch: the head's Q slice, the wave's first query
@@ -445,11 +449,11 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 // clamped to the last real row (rows past the end carry weight 0)
                 const char *src;
                 if (RAGGED) {
-                    const int row_in_tile = (PRE == 8) ? kg * 4 + (lane >> 4) : kg * 8 + (lane >> 3);
-                    const int in_row_b = (PRE == 8) ? (lane & 15) * 8 : (lane & 7) * 16;
+                    const int row_in_tile = (PRE == 8) ? kg * 4 + (lane >> 4) : (PRE == 4) ? kg * 8 + (lane >> 3) : kg * 16 + (lane >> 2);
+                    const int in_row_b = (PRE == 8) ? (lane & 15) * 8 : (PRE == 4) ? (lane & 7) * 16 : (lane & 3) * 32;
                     src = u_qhead[ua] + (size_t)min(u_qfirst[ua] + row_in_tile, a.Sq - 1) * q_row_b + in_row_b;
                 } else {
-                    src = u_qtile[ua] + ((PRE == 8) ? kg * 512 + lane * 8 : kg * 1024 + lane * 16);
+                    src = u_qtile[ua] + ((PRE == 8) ? kg * 512 + lane * 8 : (PRE == 4) ? kg * 1024 + lane * 16 : kg * 2048 + lane * 32);
                 }
                 // Issued from inline assembly, so that the compiler does not count it among the loads
                 // it waits for itself: it cannot tell how many DMA fetches were issued behind this
@@ -457,6 +461,7 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 // for exactly this load.
                 if (PRE == 8) asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(qraw) : "v"(src) : "memory");
                 else asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qraw) : "v"(src) : "memory");
+                if (PRE == 2) asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(qraw_hi) : "v"(src) : "memory");
             }
         } else if (j == 0)
             fetch_piece(u_qtile[ua], q_voff, slot, tt);
@@ -495,30 +500,39 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     auto q_publish = [&](int buf, auto behind_c) {
         // the raw rows have landed once at most the DMA instructions requested behind them are
         // outstanding (a compile-time count)
-        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(qraw) : "n"(decltype(behind_c)::value) : "memory");
-        half8 sc = kZero8;
-        if (QS) {
-            const float cs = a.negate ? -a.c : a.c;
-            typedef _Float16 qhalf_t __attribute__((ext_vector_type(PRE == 8 ? 4 : 8)));
-            const qhalf_t raw = __builtin_bit_cast(qhalf_t, qraw);
+        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(qraw), "+v"(qraw_hi) : "n"(decltype(behind_c)::value) : "memory");
+        // 16 bytes of raw rows -> 16 bytes to publish: scaled by c (sign included) in fp32 and rounded to
+        // fp16, or (QS = false) as they are with only the scale's sign applied to the sign bits
+        auto prepared = [&](qraw_t raw_w) {
+            half8 sc = kZero8;
+            if (QS) {
+                const float cs = a.negate ? -a.c : a.c;
+                typedef _Float16 qhalf_t __attribute__((ext_vector_type(PRE == 8 ? 4 : 8)));
+                const qhalf_t raw = __builtin_bit_cast(qhalf_t, raw_w);
 #pragma unroll
-            for (int e = 0; e < (PRE == 8 ? 4 : 8); ++e) sc[e] = (_Float16)((float)raw[e] * cs);
-        } else {
-            // shared as it is: only the sign bit of every 16-bit value (fp16 and bf16 alike) follows the scale's sign
-            uint4v u = {0u, 0u, 0u, 0u};
-            const uint32_t flip = a.negate ? 0x80008000u : 0u;
+                for (int e = 0; e < (PRE == 8 ? 4 : 8); ++e) sc[e] = (_Float16)((float)raw[e] * cs);
+            } else {
+                uint4v u = {0u, 0u, 0u, 0u};
+                const uint32_t flip = a.negate ? 0x80008000u : 0u;
 #pragma unroll
-            for (int e = 0; e < (PRE == 8 ? 2 : 4); ++e) u[e] = qraw[e] ^ flip;
-            sc = __builtin_bit_cast(half8, u);
-        }
+                for (int e = 0; e < (PRE == 8 ? 2 : 4); ++e) u[e] = raw_w[e] ^ flip;
+                sc = __builtin_bit_cast(half8, u);
+            }
+            return sc;
+        };
+        const half8 sc = prepared(qraw);
         char *tile = qshare + (buf * PQG + qg) * 4096;
         if (PRE == 8) {  // 4 rows per wave, 8 bytes per lane
             const int row = kg * 4 + (lane >> 4), pc = (lane & 15) >> 1, hf = lane & 1;
             const uint4v u = __builtin_bit_cast(uint4v, sc);
             *reinterpret_cast<uint2 *>(tile + row * 128 + ((pc ^ ((row >> 1) & 7)) * 16) + hf * 8) = uint2{u[0], u[1]};
-        } else {         // 8 rows per wave, one whole 16-byte piece per lane
+        } else if (PRE == 4) {  // 8 rows per wave, one whole 16-byte piece per lane
             const int row = kg * 8 + (lane >> 3), pc = lane & 7;
             *reinterpret_cast<half8 *>(tile + row * 128 + ((pc ^ ((row >> 1) & 7)) * 16)) = sc;
+        } else {  // 16 rows per wave, two adjacent pieces per lane
+            const int row = kg * 16 + (lane >> 2), pc = (lane & 3) * 2;
+            *reinterpret_cast<half8 *>(tile + row * 128 + ((pc ^ ((row >> 1) & 7)) * 16)) = sc;
+            *reinterpret_cast<half8 *>(tile + row * 128 + (((pc + 1) ^ ((row >> 1) & 7)) * 16)) = prepared(qraw_hi);
         }
     };
     auto take_q_shared = [&](int buf, half8 (&dst)[NT]) {
@@ -637,12 +651,14 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 if (t + NS < TPW) fetch_key_tile(0, tile_of(t + NS), slot_of_step(t));
                 else if (next_key_head) fetch_key_tile(1, slot_of_step(t), slot_of_step(t));
                 // The tile of step t + 1 (t + 1 >= NS) was requested at step t + 1 - NS; behind it: the
-                // tiles requested at the later steps, up to step TPW - NS - 1, and the Q rows at step TQ.
+                // tiles requested at the steps after that one, up to this step or step TPW - NS - 1 (the
+                // last one that requests a tile), i.e. min(NS - 1, TPW - 2 - t) tiles, and the Q rows at
+                // step TQ.
                 // (The requests for another key head are not counted: with them outstanding the waits
                 // below only wait for more than they need.)
                 if (t + 1 >= NS && t + 1 < TPW) {
-                    if (t >= TQ) FCS_WAIT_VM(1);
-                    else FCS_WAIT_VM((TPW - 2 - t) * NT);
+                    if (t >= TQ) FCS_WAIT_VM(QV);
+                    else FCS_WAIT_VM((TPW - 2 - t < NS - 1 ? TPW - 2 - t : NS - 1) * NT);
                 }
                 if (t + 1 < TPW) take_issue(slot_of_step(t + 1), kf[(t + 1) & 1]);
             } else {
@@ -809,27 +825,28 @@ static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.f_nwgq * p.B, p.f_hg);  // x = batch entry * f_nwgq + workgroup along the query axis
     const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
-    const bool pre = !BF && TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4) && (long)p.H * p.q_rows >= 4096 &&
-                     fabsf(a.c) <= 0.1251f * 1.44269504f;
-    // the other calls with five to eight tiles per wave: Q shared through LDS as it is, key-only ring
+    // shared-Q variants: five to eight tiles per wave and 8, 4 or 2 key groups (S 257 .. 2048)
     constexpr int TPWS = (TPW >= 5) ? TPW : 8;
-    const bool shared_q = !pre && TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4);
-    if (shared_q && p.f_kg == 8) {
-        hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 8, BF, false>), grid, dim3(512), 0, st, a);
-        return;
-    }
-    if (shared_q) {
-        hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 4, BF, false>), grid, dim3(512), 0, st, a);
-        return;
-    }
+    const bool shared_q = TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4 || p.f_kg == 2);
+    // ... pre-scaled when the rounding of Q*c to fp16 cannot show in the means
+    const bool pre = shared_q && !BF && (long)p.H * p.q_rows >= 4096 && fabsf(a.c) <= 0.1251f * 1.44269504f;
     if (pre && whole && TPW == 8 && p.f_kg == 8)
         hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 8, false>), grid, dim3(512), 0, st, a);
     else if (pre && whole && TPW == 8 && p.f_kg == 4)
         hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 4, false>), grid, dim3(512), 0, st, a);
     else if (pre && p.f_kg == 8)
-        hipLaunchKernelGGL((fcs_fused_kernel<64, (TPW >= 5 ? TPW : 8), true, 8, false>), grid, dim3(512), 0, st, a);
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 8, false>), grid, dim3(512), 0, st, a);
+    else if (pre && p.f_kg == 4)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 4, false>), grid, dim3(512), 0, st, a);
     else if (pre)
-        hipLaunchKernelGGL((fcs_fused_kernel<64, (TPW >= 5 ? TPW : 8), true, 4, false>), grid, dim3(512), 0, st, a);
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 2, false>), grid, dim3(512), 0, st, a);
+    // ... else Q shared through LDS as it is (8 or 4 key groups)
+    else if (shared_q && p.f_kg == 8)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 8, BF, false>), grid, dim3(512), 0, st, a);
+    else if (shared_q && p.f_kg == 4)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 4, BF, false>), grid, dim3(512), 0, st, a);
+    // (two key groups that cannot be pre-scaled stay on the private rings below: sharing the Q tile as
+    // it is was measured 4 % slower there, B 64 H 16 S 512 bf16 67.2 -> 69.9 us)
     else if (whole)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false, 0, BF>), grid, dim3(512), 0, st, a);
     else

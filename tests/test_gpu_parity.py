@@ -817,6 +817,12 @@ def test_fused_path_with_several_row_blocks_per_workgroup(qs, ks, kw):
     ((2, 8, 2048, 64), (2, 2, 2048, 64), {}),                       # grouped key heads: four query heads per key head
     ((2, 12, 1000, 64), (2, 4, 1536, 64), {}),                      # grouped, S_q != S_k
     ((4, 4, 1024, 64), (4, 4, 1024, 64), {"scale": -0.125}),        # two query groups per workgroup, negated scores
+    ((8, 8, 512, 64), (8, 8, 512, 64), {}),                         # two key groups: eight tiles through three slots
+    ((6, 16, 448, 64), (6, 16, 448, 64), {}),                       # two key groups, seven tiles
+    ((9, 12, 384, 64), (9, 12, 384, 64), {}),                       # two key groups, six tiles
+    ((16, 16, 300, 64), (16, 16, 300, 64), {}),                     # two key groups, five tiles, the last one moved back
+    ((3, 8, 1792, 64), (3, 8, 1792, 64), {}),                       # seven tiles through four slots
+    ((5, 16, 1100, 64), (5, 16, 1100, 64), {"scale": 0.3}),         # five tiles, Q shared as it is
 ])
 def test_key_tiles_kept_between_row_blocks(qs, ks, kw):
     """The pre-scaled fused variants with eight or six key tiles per wave leave half of a head's key
