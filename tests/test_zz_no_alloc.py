@@ -34,7 +34,7 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
 
     lib = _hip.lib()
     g = torch.Generator().manual_seed(31)
-    # larger call first (fused path, 4 MiB of slabs), then smaller ones that reuse the dirty array:
+    # larger call first (fused path, 2 MiB of slabs), then smaller ones that reuse the dirty array:
     # a ragged fused call, a two-pass call (row statistics + partials) and a few-rows call
     cases = [((8, 16, 2048, 64), -1, 0.125), ((3, 5, 333, 64), -1, 0.2), ((2, 3, 300, 128), -1, 0.1),
              ((4, 6, 577, 64), 1, 0.125), ((1, 2, 40, 64), -1, 0.125)]
