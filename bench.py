@@ -43,17 +43,8 @@ WORKLOADS = {
     "causal_h32_q128_k16384_d128": ((1, 32, 128, 128), (1, 32, 16384, 128), dict(is_causal=True), False),
     "causal_h32_q512_k65536_d128_peaky": ((1, 32, 512, 128), (1, 32, 65536, 128), dict(is_causal=True), False),
 }
-KERNELS_OF = {
-    "noncausal_b2_h4_s512_d64": "fcs_fused_kernel<64,8,false,0,false,true> + fcs_finalize_kernel<32> (one call)",
-    "noncausal_b8_h16_s2048_d64": "fcs_fused_kernel<64,8,false,8,false,true> + fcs_finalize_kernel<8> (one call; the fused kernel is >= 96 % of it)",
-    "cls1_b32_h16_s577_d64": "fcs_fewrows_kernel<64,1> + fcs_finalize_kernel<8> (one call)",
-    "noncausal_b256_h16_s1024_d64": "fcs_fused_kernel<64,8,false,4,false,true> + fcs_finalize_kernel<8> (one call)",
-    "causal_h32_q128_k4096_d128": "fcs_rowstream_kernel<128,1,4> + fcs_colstream_kernel<128,1,4> + fcs_finalize_kernel<8> (one call)",
-    "causal_h32_q128_k16384_d128": "fcs_rowstream_kernel<128,1,4> + fcs_colstream_kernel<128,1,4> + fcs_finalize_kernel<8> (one call)",
-    "causal_h32_q512_k65536_d128_peaky": "fcs_rowstream_kernel<128,2,8> + fcs_colstream_kernel<128,2,8> + fcs_finalize_kernel<8> (one call)",
-}
 DEFAULT = "noncausal_b8_h16_s2048_d64"
-SETTLE_CALLS = 150  # untimed, before the --warmup steps
+SETTLE_CALLS = 150  # untimed calls before the --warmup steps (the GPU's clocks settle under load); reported in the record
 
 
 def make_inputs(name):
@@ -178,19 +169,17 @@ def main():
     cls_n = int(kwargs.get("cls_len") or -1)
     scale = float(kwargs.get("scale") or d ** -0.5)
     lib = _hip.lib()
-    n_ws = _hip.workspace_bytes(causal, b, h, sq, sk, d, cls_n)
+    stream = torch.cuda.current_stream().cuda_stream
+    # the call as the host layer issues it: fcs_colsum_call
+    call, call_ref, n_ws = _hip._prepared_call(causal, q, k, scale, cls_n, max(0, sk - sq) if causal else 0)
     ws = torch.empty(max(n_ws, 1), dtype=torch.uint8, device="cuda")
     out = torch.empty((b, sk), dtype=torch.float32, device="cuda")
-    qs_, ks_ = _hip._I64x4(*q.stride()), _hip._I64x4(*k.stride())
-    stream = torch.cuda.current_stream().cuda_stream
+    call.q, call.k, call.out, call.out_f16 = q.data_ptr(), k.data_ptr(), out.data_ptr(), None
+    call.ws, call.ws_bytes, call.hip_stream = ws.data_ptr(), n_ws, stream
+    plan_text = _hip.plan_description(q.shape, k.shape, causal=causal, cls_n=cls_n, scale=scale)
 
     def launch():
-        if causal:
-            rc = lib.fcs_colsum_causal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), None, ws.data_ptr(), n_ws,
-                                           h, sq, sk, d, max(0, sk - sq), qs_, ks_, scale, stream)
-        else:
-            rc = lib.fcs_colsum_noncausal_f16(q.data_ptr(), k.data_ptr(), out.data_ptr(), None, ws.data_ptr(), n_ws,
-                                              b, h, sq, d, qs_, ks_, scale, cls_n, stream)
+        rc = lib.fcs_colsum_call(call_ref)
         if rc != 0:
             raise RuntimeError(_hip.strerror(rc))
 
@@ -214,7 +203,7 @@ def main():
     ker_gbs = by / (ker_ms * 1e-3) / 1e9
     roofline = {
         "bound": "mfma",
-        "kernel": KERNELS_OF[name],
+        "kernel": plan_text + " (all kernels of one call)",
         "achieved": round(ker_tflops, 2),
         "peak": PEAK_FP16_TFLOPS,
         "unit": "TFLOP/s",
@@ -285,6 +274,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_calls": SETTLE_CALLS,
         "ms_per_step": round(ms_call, 5),
         "ms_per_call_synced": round(ms_call_synced, 5),
         "value_synced": round(fl / (ms_call_synced * 1e-3) / 1e12, 2),

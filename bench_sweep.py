@@ -15,7 +15,11 @@ then `iters` x (call + device synchronize) under one wall clock, so launch and h
 are included.  Peak memory is `torch.cuda.max_memory_allocated` around one call
 (benchmark_colsum.py:59-71); the kernels' workspace is allocated once per stream by the host
 layer and reported in its own column.  The eager baseline that materialises the attention matrix runs
-on the GPU too, and is skipped (empty CSV fields) when its score tensors would not fit.
+on the GPU too.  Where its score tensors would not fit it runs in chunks (`eager_kind` says how), each
+chunk the same eager code on a slice: over the batch for the batched sweep, over query rows elsewhere
+(a row's softmax needs all keys, so rows are what can be cut).  The reference's benchmark has the same
+fallback (benchmarks/benchmark_colsum.py:74-196, 234-274; it estimates the batched case from the largest
+batch that fitted, here it is run).
 
     python bench_sweep.py --sweep all --out sweep.csv
 """
@@ -65,6 +69,40 @@ def peak_memory(fn):
     return torch.cuda.max_memory_allocated() - base
 
 
+def chunked_eager(naive_colsum, q, k, scale, causal, budget_bytes):
+    """The eager baseline on slices that fit `budget_bytes` of score tensors; returns (fn, kind, chunk).
+
+    Batch > 1: slices of the batch (results concatenated).  Batch 1: slices of query rows; a slice's means
+    are weighted by its rows and added (causal: rows [r0, r1) see the keys below k_past + r1 and are aligned
+    to the end of that prefix, which is the alignment the eager code infers from the shapes)."""
+    import torch
+
+    b, h, sq, _ = q.shape
+    sk = k.shape[2]
+    per_score = 2 + 4 + 2 + 2  # logits, fp32 softmax, its cast, one temporary
+    if b > 1:
+        chunk = max(1, min(b, budget_bytes // (h * sq * sk * per_score)))
+
+        def fn():
+            return torch.cat([naive_colsum(q[i:i + chunk], k[i:i + chunk], scale=scale, is_causal=causal)
+                              for i in range(0, b, chunk)], dim=0)
+        return fn, "chunked_batch", chunk
+    chunk = max(1, min(sq, budget_bytes // (h * sk * per_score)))
+    k_past = max(0, sk - sq) if causal else 0
+
+    def fn():
+        out = torch.zeros((1, sk), dtype=torch.float32, device=q.device)
+        for r0 in range(0, sq, chunk):
+            r1 = min(sq, r0 + chunk)
+            if causal:
+                part = naive_colsum(q[:, :, r0:r1], k[:, :, :k_past + r1], scale=scale, is_causal=True)
+                out[:, :k_past + r1] += part.float() * (r1 - r0)
+            else:
+                out += naive_colsum(q[:, :, r0:r1], k, scale=scale).float() * (r1 - r0)
+        return out / sq
+    return fn, "chunked_rows", chunk
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--sweep", default="all", choices=sorted(SWEEPS) + ["all"])
@@ -82,7 +120,7 @@ def main():
         sys.exit("bench_sweep.py needs a GPU")
     names = sorted(SWEEPS) if args.sweep == "all" else [args.sweep]
     fields = ["sweep", "B", "H", "Sq", "Sk", "D", "causal", "flash_ms", "flash_peak_mib", "workspace_mib", "flash_tflops",
-              "eager_ms", "eager_peak_mib", "speedup", "max_abs_diff_vs_eager"]
+              "eager_ms", "eager_peak_mib", "speedup", "max_abs_diff_vs_eager", "eager_kind", "eager_chunk"]
     out = sys.stdout if args.out == "-" else open(args.out, "w", newline="")
     wr = csv.DictWriter(out, fieldnames=fields)
     wr.writeheader()
@@ -106,10 +144,16 @@ def main():
                        flash_tflops=round(4.0 * pt["B"] * pt["H"] * pt["Sq"] * pt["Sk"] * pt["D"] / t_fast / 1e12, 1),
                        **{f: pt[f] for f in ("B", "H", "Sq", "Sk", "D")})
             scores = pt["B"] * pt["H"] * pt["Sq"] * pt["Sk"]
-            if not args.no_eager and scores * (2 + 4 + 2 + 2) <= EAGER_MAX_BYTES:
-                ref = lambda: naive_colsum(q, k, scale=scale, is_causal=pt["causal"])
+            if not args.no_eager:
+                if scores * (2 + 4 + 2 + 2) <= EAGER_MAX_BYTES:
+                    ref, kind, chunk = (lambda: naive_colsum(q, k, scale=scale, is_causal=pt["causal"])), "full", ""
+                else:
+                    ref, kind, chunk = chunked_eager(naive_colsum, q, k, scale, pt["causal"], EAGER_MAX_BYTES // 2)
+                row.update(eager_kind=kind, eager_chunk=chunk)
                 try:
-                    t_ref = measure_latency(ref, 1, max(3, min(iters, int(1.0 / max(t_fast * 20, 1e-6)) or 3)))
+                    t_probe_ref = measure_latency(ref, 0, 1)  # long points: one warm-up is the probe itself
+                    n_ref = max(1, min(iters, int(2.0 / max(t_probe_ref, 1e-6))))
+                    t_ref = t_probe_ref if n_ref == 1 and t_probe_ref > 2.0 else measure_latency(ref, 0, max(n_ref, 2))
                     m_ref = peak_memory(ref)
                     diff = (run().float() - ref().float()).abs().max().item()
                     row.update(eager_ms=round(t_ref * 1e3, 4), eager_peak_mib=round(m_ref / 2**20, 2),

@@ -65,17 +65,22 @@ static constexpr int kDppMirror = 0x140;      // lane i <-> 15 - i within rows o
 // run on one XCD and close together in time.  This returns the grid coordinates a workgroup should
 // work on instead of its own: XCD c, which receives workgroups c, c + 8, c + 16, ..., then walks a
 // contiguous range of the x-fastest list of all coordinates.  A bijection for any grid size.
-__device__ __forceinline__ void xcd_contiguous_block(int &bx, int &by, int &bz)
+// `i` is the workgroup's number in launch order, nx * ny * nz the number of workgroups.
+__device__ __forceinline__ void xcd_contiguous_block(int i, int nx, int ny, int nz, int &bx, int &by, int &bz)
 {
-    const int nx = gridDim.x, ny = gridDim.y;
-    const int n_all = nx * ny * (int)gridDim.z;
-    const int i = ((int)blockIdx.z * ny + (int)blockIdx.y) * nx + (int)blockIdx.x;
+    const int n_all = nx * ny * nz;
     const int c = i & 7, per = n_all >> 3, rem = n_all & 7;  // XCD c holds per + (c < rem) workgroups
     const int v = c * per + min(c, rem) + (i >> 3);
     bx = v % nx;
     const int t = v / nx;
     by = t % ny;
     bz = t / ny;
+}
+// the same for a kernel whose grid is (nx, ny, nz)
+__device__ __forceinline__ void xcd_contiguous_block(int &bx, int &by, int &bz)
+{
+    const int nx = gridDim.x, ny = gridDim.y;
+    xcd_contiguous_block(((int)blockIdx.z * ny + (int)blockIdx.y) * nx + (int)blockIdx.x, nx, ny, (int)gridDim.z, bx, by, bz);
 }
 
 }  // namespace fcs

@@ -13,6 +13,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <stdio.h>
+
 #include "fcs_device.h"
 #include "fcs_kernels.h"
 #include "fcs_plan.h"
@@ -164,6 +166,15 @@ hipError_t launch_fewrows(const Plan &p, const Args &a, hipStream_t st)
         e = (p.D == 64) ? launch_fewrows_d<64, false>(p, a, st) : launch_fewrows_d<128, false>(p, a, st);
     if (e != hipSuccess) return e;
     return launch_finalize(a, st);
+}
+
+size_t describe_fewrows(const Plan &p, const Args &a, char *buf, size_t n)
+{
+    const int r = snprintf(buf, n, "fcs_fewrows_kernel<%d,%d,%s> grid %d, %d heads per workgroup, %d slabs", p.D, p.q_rows,
+                           p.bf16 ? "true" : "false", p.B * p.f_hg, p.f_hpg, p.n_partials);
+    if (r < 0) return 0;
+    const size_t len = (size_t)r;
+    return len + describe_finalize(a, len < n ? buf + len : nullptr, len < n ? n - len : 0);
 }
 
 }  // namespace fcs

@@ -30,6 +30,8 @@
 
 #include <type_traits>
 
+#include <stdio.h>
+
 #include "fcs_device.h"
 #include "fcs_kernels.h"
 
@@ -820,37 +822,65 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     }
 }
 
+// Which instantiation serves a call with TPW key tiles per wave (shared by the launcher and the plan description).
+struct FusedVariant {
+    int tpw;      // template TPW (the shared-Q variants exist for five to eight tiles)
+    bool ragged;
+    int pre;      // 8, 4, 2: shared Q tile with that many key groups; 0: private rings
+    bool qs;      // shared Q tile pre-scaled
+};
+static FusedVariant pick_fused(const Plan &p, const Args &a, bool bf)
+{
+    const int TPW = p.f_tpw;
+    const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
+    // shared-Q variants: five to eight tiles per wave and 8, 4 or 2 key groups (S 257 .. 2048)
+    const bool shared_q = TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4 || p.f_kg == 2);
+    // ... pre-scaled when the rounding of Q*c to fp16 cannot show in the means
+    const bool pre = shared_q && !bf && (long)p.H * p.q_rows >= 4096 && fabsf(a.c) <= 0.1251f * 1.44269504f;
+    if (pre && whole && TPW == 8 && (p.f_kg == 8 || p.f_kg == 4)) return {8, false, p.f_kg, true};
+    if (pre) return {TPW, true, p.f_kg, true};
+    // ... else Q shared through LDS as it is (8 or 4 key groups).  (Two key groups that cannot be
+    // pre-scaled stay on the private rings: sharing the Q tile as it is was measured 4 % slower there,
+    // B 64 H 16 S 512 bf16 67.2 -> 69.9 us.)
+    if (shared_q && p.f_kg != 2) return {TPW, true, p.f_kg, false};
+    return {TPW, !whole, 0, true};
+}
+
 template <int TPW, bool BF>
 static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 {
     const dim3 grid(p.f_nwgq * p.B, p.f_hg);  // x = batch entry * f_nwgq + workgroup along the query axis
-    const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
-    // shared-Q variants: five to eight tiles per wave and 8, 4 or 2 key groups (S 257 .. 2048)
     constexpr int TPWS = (TPW >= 5) ? TPW : 8;
-    const bool shared_q = TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4 || p.f_kg == 2);
-    // ... pre-scaled when the rounding of Q*c to fp16 cannot show in the means
-    const bool pre = shared_q && !BF && (long)p.H * p.q_rows >= 4096 && fabsf(a.c) <= 0.1251f * 1.44269504f;
-    if (pre && whole && TPW == 8 && p.f_kg == 8)
+    const FusedVariant v = pick_fused(p, a, BF);
+    if (v.pre == 8 && v.qs && !v.ragged)
         hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 8, false>), grid, dim3(512), 0, st, a);
-    else if (pre && whole && TPW == 8 && p.f_kg == 4)
+    else if (v.pre == 4 && v.qs && !v.ragged)
         hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 4, false>), grid, dim3(512), 0, st, a);
-    else if (pre && p.f_kg == 8)
+    else if (v.pre == 8 && v.qs)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 8, false>), grid, dim3(512), 0, st, a);
-    else if (pre && p.f_kg == 4)
+    else if (v.pre == 4 && v.qs)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 4, false>), grid, dim3(512), 0, st, a);
-    else if (pre)
+    else if (v.pre == 2 && v.qs)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 2, false>), grid, dim3(512), 0, st, a);
-    // ... else Q shared through LDS as it is (8 or 4 key groups)
-    else if (shared_q && p.f_kg == 8)
+    else if (v.pre == 8)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 8, BF, false>), grid, dim3(512), 0, st, a);
-    else if (shared_q && p.f_kg == 4)
+    else if (v.pre == 4)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPWS, true, 4, BF, false>), grid, dim3(512), 0, st, a);
-    // (two key groups that cannot be pre-scaled stay on the private rings below: sharing the Q tile as
-    // it is was measured 4 % slower there, B 64 H 16 S 512 bf16 67.2 -> 69.9 us)
-    else if (whole)
+    else if (!v.ragged)
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, false, 0, BF>), grid, dim3(512), 0, st, a);
     else
         hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true, 0, BF>), grid, dim3(512), 0, st, a);
+}
+
+size_t describe_fused(const Plan &p, const Args &a, char *buf, size_t n)
+{
+    const FusedVariant v = pick_fused(p, a, p.bf16 != 0);
+    int r = snprintf(buf, n, "fcs_fused_kernel<64,%d,%s,%d,%s,%s> grid %d x %d, %d x %d units per workgroup, %d slabs", v.tpw,
+                     v.ragged ? "true" : "false", v.pre, (p.bf16 && !(v.pre && v.qs)) ? "true" : "false", v.qs ? "true" : "false",
+                     p.f_nwgq * p.B, p.f_hg, p.f_hpg, p.f_rbpw, p.n_partials);
+    if (r < 0) return 0;
+    const size_t len = (size_t)r;
+    return len + describe_finalize(a, len < n ? buf + len : nullptr, len < n ? n - len : 0);
 }
 
 template <bool BF>

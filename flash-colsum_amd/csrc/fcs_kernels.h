@@ -27,6 +27,8 @@ struct Args {
     float2 *ml;   // [B*H][n_chunks][rows_pad]  (m, l) of each key split
     // pass 2
     int c_chunk, c_groups, c_upg, c_nrb;  // column pass: keys per block, unit groups, units per group, row blocks per head
+    int c_nchunks;       // column pass: key chunks (its grid is c_nchunks x c_groups x B, launched as one dimension)
+    int n_qblk;          // pass 1: row blocks (its grid is n_qblk x n_chunks x B*H, launched as one dimension)
     float *partial;  // [groups][B][Sk]
     float *out;      // [B][Sk]
     _Float16 *out_h; // [B][Sk] or nullptr: the same means rounded to fp16
@@ -39,6 +41,7 @@ struct Args {
     int f_hpg;       // heads per block
     int f_rbpw;      // adjacent row blocks per block (a block walks over f_rbpw x f_hpg units)
     int f_nwgq;      // blocks along the query axis: ceil(f_nqblk / f_rbpw)
+    int f_hg;        // head groups (fused and few-rows paths): a batch entry has f_hg * f_nwgq workgroups
 };
 
 // Enqueues every kernel of one call on `stream`; returns 0 or the hipError_t of a failed launch.
@@ -55,5 +58,12 @@ hipError_t launch_colstream(const Plan &p, const Args &a, hipStream_t st);
 
 // shared final reduction out = inv_norm * sum of the n_partials slabs (fcs_kernels.hip)
 hipError_t launch_finalize(const Args &a, hipStream_t st);
+
+// Text description of what launch_colsum(p, a, .) launches; snprintf semantics.
+size_t describe_colsum(const Plan &p, const Args &a, char *buf, size_t n);
+size_t describe_fused(const Plan &p, const Args &a, char *buf, size_t n);
+size_t describe_fewrows(const Plan &p, const Args &a, char *buf, size_t n);
+size_t describe_two_pass(const Plan &p, const Args &a, char *buf, size_t n);
+size_t describe_finalize(const Args &a, char *buf, size_t n);
 
 }  // namespace fcs

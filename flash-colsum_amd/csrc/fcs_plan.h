@@ -52,6 +52,7 @@ struct Plan {
     int f_rbpw;      // adjacent query blocks per workgroup (fused path; 1 on the few-rows path)
     int f_nwgq;      // workgroups along the query axis: ceil(f_nqblk / f_rbpw)
     int n_partials;  // slabs summed by the finalize kernel
+    int gen_blocks;  // two-pass path: resident workgroups of one generation (what the GPU holds at once)
     // workspace layout (byte offsets, each 256-byte aligned)
     size_t off_lse;      // float2 [B*H][rows_pad]            row maximum and log2 of the row sum
     size_t off_ml;       // float2 [B*H][n_chunks][rows_pad]  only when n_chunks > 1
@@ -93,7 +94,9 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     // One generation of workgroups: an 8-wave block fills a compute unit's registers, the 4-wave
     // blocks fit twice.  Every further generation pays the block start (Q fragments, first key
     // stage: ~5 us) again, which nothing overlaps.
-    const int target1 = (p.k1_waves == 8) ? kComputeUnits : 2 * kComputeUnits;
+    // (256-wide heads: the kernels' registers and LDS allow one block per compute unit whatever its waves)
+    const int target1 = (p.k1_waves == 8 || p.Dp == 256) ? kComputeUnits : 2 * kComputeUnits;
+    p.gen_blocks = target1;
     // as many splits as still fit one generation (rounding up could start a second one for a few blocks)
     int want = (base1 >= target1) ? 1 : (int)(target1 / base1);
     int max_chunks = ceil_div(Sk, 4 * kStageKeys);  // at least 256 keys per split
@@ -112,7 +115,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         p.c_nrb = ceil_div(p.q_rows, block_rows);
         const long units = (long)H * p.c_nrb;
         const int chunk_max = col_chunk_max(p.Dp, p.c_waves);
-        const long target = (p.c_waves == 8) ? kComputeUnits : 2 * kComputeUnits;
+        const long target = (p.c_waves == 8 || p.Dp == 256) ? kComputeUnits : 2 * kComputeUnits;
         int chunk = ceil_div(Sk, kStageKeys) * kStageKeys;
         if (chunk > chunk_max) chunk = chunk_max;
         int nchunks = ceil_div(Sk, chunk);
@@ -179,7 +182,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         p.n_partials = p.f_hg;
         p.off_lse = p.off_ml = p.off_partial = 0;
         p.total = align256(sizeof(float) * (size_t)p.n_partials * B * Sk);
-        return true;
+        return (long)B * p.f_hg < (1L << 31);
     }
 
     // ---- fused path
@@ -207,9 +210,9 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         for (int rbpw = 1; rbpw <= 16 && (rbpw == 1 || rbpw <= p.f_nqblk); ++rbpw) {
             const int nwgq = ceil_div(p.f_nqblk, rbpw);
             if (ceil_div(p.f_nqblk, nwgq) != rbpw) continue;  // same grouping as a smaller rbpw
-            for (int hpg = H; hpg >= 1; --hpg) {
-                const int hg = ceil_div(H, hpg);
-                if (ceil_div(H, hg) != hpg) continue;  // same grouping as a smaller hpg
+            // heads per workgroup, descending, one value per distinct grouping: hpg = ceil(H / hg) for
+            // hg = 1, then the next hg that lowers it (about 2 sqrt(H) values)
+            for (int hg = 1, hpg = H; hpg >= 1; hg = (hpg > 1) ? ceil_div(H, hpg - 1) : H + 1, hpg = (hg <= H) ? ceil_div(H, hg) : 0) {
                 const long gens = ((long)nwgq * B * hg + kComputeUnits - 1) / kComputeUnits;
                 // a unit that follows another row block of the same head finds half of its key tiles in
                 // the LDS ring (the shared-Q kernels; measured 4 % of a unit): row blocks per head count
@@ -232,10 +235,9 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         p.f_hg = ceil_div(H, p.f_hpg);
         p.f_nwgq = ceil_div(p.f_nqblk, p.f_rbpw);
         p.n_partials = p.f_hg * p.f_nwgq * p.f_qg;
-        size_t off = align256(sizeof(float) * (size_t)p.n_partials * B * Sk);
         p.off_lse = p.off_ml = p.off_partial = 0;
-        p.total = off;
-        return true;
+        p.total = align256(sizeof(float) * (size_t)p.n_partials * B * Sk);
+        return (long)p.f_nwgq * B * p.f_hg < (1L << 31);
     }
 
     // ---- workspace
@@ -247,7 +249,8 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     p.off_partial = off;
     if (p.c_groups > 1) off = align256(off + sizeof(float) * (size_t)p.c_groups * B * Sk);
     p.total = off;
-    return true;
+    // both passes launch one-dimensional grids
+    return (long)p.n_qblk * p.n_chunks * B * H < (1L << 31) && (long)p.c_nchunks * p.c_groups * B < (1L << 31);
 }
 
 }  // namespace fcs

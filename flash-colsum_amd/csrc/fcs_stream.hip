@@ -32,6 +32,8 @@
 
 #include <type_traits>
 
+#include <stdio.h>
+
 #include "fcs_device.h"
 #include "fcs_kernels.h"
 
@@ -121,7 +123,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int cx, grp, b;  // chunks of one (group, batch entry) stream the same Q: neighbours in launch order
-    xcd_contiguous_block(cx, grp, b);
+    xcd_contiguous_block((int)blockIdx.x, a.c_nchunks, a.c_groups, a.B, cx, grp, b);  // a one-dimensional grid: no axis limit
     const int c0 = cx * a.c_chunk;                     // first key of the chunk
     const int c1 = min(a.Sk, c0 + a.c_chunk);          // one past its last key
     const int u_begin = grp * a.c_upg, u_end = min(a.H * a.c_nrb, u_begin + a.c_upg);
@@ -519,7 +521,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int bx, chunk, bh;  // row blocks of one (key split, head) read the same keys: same XCD
-    xcd_contiguous_block(bx, chunk, bh);
+    xcd_contiguous_block((int)blockIdx.x, a.n_qblk, a.n_chunks, a.B * a.H, bx, chunk, bh);  // a one-dimensional grid: no axis limit
     const int b = bh / a.H, h = bh - b * a.H;
     const int row0 = bx * BLOCK_ROWS, qw0 = row0 + wave * ROWS_W;
     const float cmul = a.c;
@@ -796,7 +798,7 @@ static bool stream_prescaled(const Plan &p, const Args &a)
 template <int D, int NB, int WAVES, bool BF>
 static hipError_t launch_cfg(const Plan &p, const Args &a, hipStream_t st)
 {
-    const dim3 grid(p.c_nchunks, p.c_groups, p.B);
+    const dim3 grid((unsigned)((long)p.c_nchunks * p.c_groups * p.B));
     if constexpr (D == 64 && !BF) {
         if (stream_prescaled(p, a)) {
             hipLaunchKernelGGL((fcs_colstream_kernel<D, NB, WAVES, BF, true>), grid, dim3(64 * WAVES), 0, st, a);
@@ -824,7 +826,7 @@ static hipError_t launch_colstream_d(const Plan &p, const Args &a, hipStream_t s
 template <int D, int NB, int WAVES, bool BF>
 static hipError_t launch_rows_cfg(const Plan &p, const Args &a, hipStream_t st)
 {
-    const dim3 grid(p.n_qblk, p.n_chunks, p.B * p.H);
+    const dim3 grid((unsigned)((long)p.n_qblk * p.n_chunks * p.B * p.H));
     if constexpr (D == 64 && !BF) {
         if (stream_prescaled(p, a)) {
             hipLaunchKernelGGL((fcs_rowstream_kernel<D, NB, WAVES, BF, true>), grid, dim3(64 * WAVES), 0, st, a);
@@ -844,6 +846,21 @@ static hipError_t launch_rowstream_d(const Plan &p, const Args &a, hipStream_t s
     }
     if (p.qw == 32 && p.k1_waves == 4) return launch_rows_cfg<D, 1, 4, BF>(p, a, st);
     return hipErrorInvalidValue;
+}
+
+size_t describe_two_pass(const Plan &p, const Args &a, char *buf, size_t n)
+{
+    const bool pre = stream_prescaled(p, a);
+    const int nb1 = p.qw / 32;
+    int r = snprintf(buf, n,
+                     "fcs_rowstream_kernel<%d,%d,%d,%s,%s> grid %d x %d x %d + fcs_colstream_kernel<%d,%d,%d,%s,%s> grid %d x %d x %d, "
+                     "%d units per workgroup",
+                     p.Dp, nb1, p.k1_waves, p.bf16 ? "true" : "false", pre ? "true" : "false", p.n_qblk, p.n_chunks, p.B * p.H, p.Dp,
+                     p.c_nb, p.c_waves, p.bf16 ? "true" : "false", pre ? "true" : "false", p.c_nchunks, p.c_groups, p.B, p.c_upg);
+    if (r < 0) return 0;
+    const size_t len = (size_t)r;
+    if (p.c_groups > 1) return len + describe_finalize(a, len < n ? buf + len : nullptr, len < n ? n - len : 0);
+    return len;
 }
 
 hipError_t launch_rowstream(const Plan &p, const Args &a, hipStream_t st)

@@ -62,6 +62,8 @@ __device__ __forceinline__ int block_rank(bool flag, int *wsum, int &total)
 
 // taken elements of one row in ascending index order.  thr_key: elements with a larger key are taken;
 // `need` more with an equal key (lowest indices first).  Returns the number written (<= cap).
+// CANON: -0 counts as +0 (the value comparison `>=` of the threshold form, not the bit order of top-k).
+template <bool CANON>
 __device__ int compact_row(const float *row, int S, uint32_t thr_key, int need, int64_t *idx_out, float *val_out, int cap,
                            int *wsum)
 {
@@ -73,7 +75,7 @@ __device__ int compact_row(const float *row, int S, uint32_t thr_key, int need, 
         const bool in = i < S;
         if (in) {
             v = row[i];
-            key = order_key(v);
+            key = order_key(CANON ? v + 0.0f : v);
         }
         const bool eq = in && key == thr_key;
         int eq_tot;
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(kTopkThreads) void fcs_topk_kernel(const float *mea
     // `prefix` is the k-th largest key; `want` of the elements equal to it are taken
 
     // ---- 2. ordered compaction
-    compact_row(row, S, prefix, want, io, vo ? vo : nullptr, k, wsum);
+    compact_row<false>(row, S, prefix, want, io, vo ? vo : nullptr, k, wsum);
 
     // ---- 3. descending values, ties by ascending index
     if (sorted && k <= kTopkSortMax) {
@@ -159,9 +161,9 @@ __global__ __launch_bounds__(kTopkThreads) void fcs_topk_kernel(const float *mea
             if (i < k) {
                 si[i] = (int)io[i];
                 sv[i] = row[io[i]];
-            } else {  // padding sorts last
+            } else {  // padding (recognised by its index) sorts behind every real entry, negative NaNs included
                 si[i] = 0x7fffffff;
-                sv[i] = -INFINITY;
+                sv[i] = 0.f;
             }
         }
         __syncthreads();
@@ -172,7 +174,8 @@ __global__ __launch_bounds__(kTopkThreads) void fcs_topk_kernel(const float *mea
                     const int lo = 2 * t - (t & (stride - 1));  // index with the `stride` bit clear
                     const int hi = lo + stride;
                     const bool desc_block = ((lo & size) == 0);  // this block ends up in "before" order
-                    const uint32_t ka = order_key(sv[lo]), kb = order_key(sv[hi]);
+                    const uint32_t ka = (si[lo] == 0x7fffffff) ? 0u : order_key(sv[lo]);
+                    const uint32_t kb = (si[hi] == 0x7fffffff) ? 0u : order_key(sv[hi]);
                     const bool a_first = ka > kb || (ka == kb && si[lo] < si[hi]);
                     if (a_first != desc_block) {
                         const float tv = sv[lo];
@@ -198,9 +201,9 @@ __global__ __launch_bounds__(kTopkThreads) void fcs_threshold_kernel(const float
 {
     __shared__ int wsum[kTopkWaves + 1];
     const float *row = means + (int64_t)blockIdx.x * S;
-    // value >= tau  <=>  key >= key(tau): take keys above key(tau) - 1 ... expressed as "larger than thr, or equal
-    // to thr with unlimited ties" with thr = key(tau)
-    const int n = compact_row(row, S, order_key(tau), 0x7fffffff, idx_out + (int64_t)blockIdx.x * S, nullptr, S, wsum);
+    // value >= tau  <=>  key(value) >= key(tau) once -0 is read as +0 on both sides (the bit order alone puts
+    // -0 below +0): "larger than thr, or equal to thr with unlimited ties" with thr = key(tau + 0)
+    const int n = compact_row<true>(row, S, order_key(tau + 0.0f), 0x7fffffff, idx_out + (int64_t)blockIdx.x * S, nullptr, S, wsum);
     if (threadIdx.x == 0) count_out[blockIdx.x] = n;
 }
 

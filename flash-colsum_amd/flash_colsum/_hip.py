@@ -18,11 +18,26 @@ from typing import Optional
 import torch
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libflashcolsum.so")
-_ABI_VERSION = 4
+_ABI_VERSION = 5
 _lib = None
 
 _I64x4 = ctypes.c_int64 * 4
 _MAX_HEAD_DIM = 256  # the library takes any multiple of 8 up to this
+
+
+class _Call(ctypes.Structure):
+    """fcs_call_t of include/flash_colsum.h: one call as a struct, filled once per tensor geometry."""
+    _fields_ = [
+        ("struct_bytes", ctypes.c_uint32), ("flags", ctypes.c_uint32),
+        ("dtype", ctypes.c_int32), ("causal", ctypes.c_int32),
+        ("B", ctypes.c_int32), ("Hq", ctypes.c_int32), ("Hk", ctypes.c_int32),
+        ("Sq", ctypes.c_int32), ("Sk", ctypes.c_int32), ("D", ctypes.c_int32),
+        ("cls_n", ctypes.c_int32), ("k_past", ctypes.c_int32),
+        ("scale", ctypes.c_float), ("reserved", ctypes.c_int32),
+        ("q_strides", _I64x4), ("k_strides", _I64x4),
+        ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("out", ctypes.c_void_p), ("out_f16", ctypes.c_void_p),
+        ("ws", ctypes.c_void_p), ("ws_bytes", ctypes.c_size_t), ("hip_stream", ctypes.c_void_p),
+    ]
 
 
 def lib() -> ctypes.CDLL:
@@ -66,6 +81,12 @@ def lib() -> ctypes.CDLL:
             ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
             ctypes.c_void_p, ctypes.c_size_t] + [ctypes.c_int] * 8 + [
             ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64), ctypes.c_float, ctypes.c_void_p]
+        cdll.fcs_colsum_call.restype = ctypes.c_int
+        cdll.fcs_colsum_call.argtypes = [ctypes.POINTER(_Call)]
+        cdll.fcs_plan_describe.restype = ctypes.c_size_t
+        cdll.fcs_plan_describe.argtypes = [ctypes.POINTER(_Call), ctypes.c_char_p, ctypes.c_size_t]
+        cdll.fcs_static_scratch_init.restype = ctypes.c_int
+        cdll.fcs_static_scratch_init.argtypes = []
         cdll.fcs_topk_f32.restype = ctypes.c_int
         cdll.fcs_topk_f32.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                       ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
@@ -92,8 +113,10 @@ def _as_kernel_input(t: torch.Tensor, dtype: torch.dtype = torch.float16) -> tor
     """`dtype` (fp16 or bf16), unit last stride, 16-byte aligned rows/heads/base; copies only when it must."""
     if t.dtype != dtype:
         t = t.to(dtype)
-    if t.is_contiguous() and t.shape[-1] % 8 == 0 and t.data_ptr() % 16 == 0:
-        return t  # the common case, decided without looking at the strides one by one
+    if t.is_contiguous() and t.shape[-1] % 8 == 0 and t.data_ptr() % 16 == 0 and t.shape[1] > 1 and t.shape[2] > 1:
+        # the common case, decided without looking at the strides one by one (a dimension of size 1 may carry
+        # any stride and still count as contiguous: those tensors take the checks below)
+        return t
     ok = (
         t.stride(3) == 1
         and t.stride(2) % 8 == 0
@@ -101,7 +124,16 @@ def _as_kernel_input(t: torch.Tensor, dtype: torch.dtype = torch.float16) -> tor
         and (t.shape[0] == 1 or t.stride(0) % 8 == 0)
         and t.data_ptr() % 16 == 0
     )
-    return t if ok else t.contiguous()
+    if ok:
+        return t
+    if not t.is_contiguous():
+        t = t.contiguous()
+    elif t.data_ptr() % 16:
+        t = t.clone()
+    # contiguous now, but the stride of a size-1 dimension may still be anything: the same memory under the
+    # dense strides
+    b, h, s_, d = t.shape
+    return t.as_strided(t.shape, (h * s_ * d, s_ * d, d, 1))
 
 
 _ws_bytes_cache = {}
@@ -117,41 +149,46 @@ def workspace_bytes(causal: bool, b: int, h: int, s_q: int, s_k: int, d: int, cl
     return n
 
 
-# One workspace per (device, stream), grown on demand and reused by later calls: calls on one
-# stream execute in order, so the next call may overwrite what the previous one left behind.
-# The cache holds at most _WS_MAX_ENTRIES streams (least recently used goes first) and nothing
+# One workspace per (thread, device, stream), grown on demand and reused by later calls: calls on one
+# stream execute in order, so the next call may overwrite what the previous one left behind; threads
+# do not share workspaces, so calls that two threads enqueue on one stream cannot meet in one either.
+# A thread keeps at most _WS_MAX_ENTRIES streams (least recently used goes first) and nothing
 # above _WS_MAX_CACHED_BYTES: larger workspaces are allocated per call and returned to torch's
 # allocator afterwards.  While a stream is capturing a HIP graph the cache is neither read nor
 # filled: the workspace then comes from the graph's own pool and lives as long as the graph.
-_workspaces = collections.OrderedDict()
-_workspaces_lock = threading.Lock()
+_tls = threading.local()
 _WS_MIN_BYTES = 1 << 20
 _WS_MAX_CACHED_BYTES = 64 << 20
 _WS_MAX_ENTRIES = 16
+_CALLS_MAX_ENTRIES = 256
 
 
 def _workspace(device: torch.device, stream: int, n_bytes: int) -> torch.Tensor:
     if n_bytes > _WS_MAX_CACHED_BYTES or torch.cuda.is_current_stream_capturing():
         return torch.empty((max(n_bytes, 256),), dtype=torch.uint8, device=device)
+    cache = getattr(_tls, "workspaces", None)
+    if cache is None:
+        cache = _tls.workspaces = collections.OrderedDict()
     key = (device.index, stream)
-    with _workspaces_lock:
-        ws = _workspaces.get(key)
-        if ws is None or ws.numel() < n_bytes:
-            ws = torch.empty((max(n_bytes, _WS_MIN_BYTES),), dtype=torch.uint8, device=device)
-            _workspaces[key] = ws
-        _workspaces.move_to_end(key)
-        while len(_workspaces) > _WS_MAX_ENTRIES:
-            _workspaces.popitem(last=False)
+    ws = cache.get(key)
+    if ws is None or ws.numel() < n_bytes:
+        ws = torch.empty((max(n_bytes, _WS_MIN_BYTES),), dtype=torch.uint8, device=device)
+        cache[key] = ws
+        while len(cache) > _WS_MAX_ENTRIES:
+            cache.popitem(last=False)
+    elif len(cache) > 1:
+        cache.move_to_end(key)
     return ws
 
 
 def release_workspaces() -> None:
-    """Drop the cached per-stream workspaces (they are otherwise kept until the process ends).
+    """Drop the calling thread's cached per-stream workspaces (they are otherwise kept until the thread ends).
 
     Kernels already enqueued keep running on the memory they were given; torch's allocator
     reuses it for later allocations on the same stream in stream order."""
-    with _workspaces_lock:
-        _workspaces.clear()
+    cache = getattr(_tls, "workspaces", None)
+    if cache is not None:
+        cache.clear()
 
 
 # the raw handle of the current stream without building a torch.cuda.Stream object (absent from some builds)
@@ -164,50 +201,58 @@ def _current_stream(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
 
-def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16, general=False, f16_only=False):
-    b, h, s_q, d = q.shape
-    s_k = k.shape[2]
+def _prepared_call(causal, q, k, scale, cls_n, k_past):
+    """The calling thread's fcs_call_t for this tensor geometry (shape, strides, dtype and the scalar
+    arguments filled in; pointers are set per call) and the workspace bytes it needs."""
+    calls = getattr(_tls, "calls", None)
+    if calls is None:
+        calls = _tls.calls = {}
+    key = (q.shape, k.shape, q.stride(), k.stride(), q.dtype, causal, cls_n, k_past, scale)
+    ent = calls.get(key)
+    if ent is None:
+        b, h, s_q, d = q.shape
+        c = _Call()
+        c.struct_bytes = ctypes.sizeof(_Call)
+        c.dtype = 1 if q.dtype == torch.bfloat16 else 0
+        c.causal = int(causal)
+        c.B, c.Hq, c.Hk, c.Sq, c.Sk, c.D = b, h, k.shape[1], s_q, k.shape[2], d
+        c.cls_n, c.k_past, c.scale = int(cls_n), int(k_past), scale
+        c.q_strides, c.k_strides = _I64x4(*q.stride()), _I64x4(*k.stride())
+        ent = (c, ctypes.byref(c), workspace_bytes(causal, b, h, s_q, k.shape[2], d, cls_n))
+        if len(calls) >= _CALLS_MAX_ENTRIES:
+            calls.clear()
+        calls[key] = ent
+    return ent
+
+
+def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16, f16_only=False):
+    c, c_ref, n_ws = _prepared_call(causal, q, k, scale, cls_n, k_past)
+    b, s_k = c.B, c.Sk
     dev = q.device
-    n_ws = workspace_bytes(causal, b, h, s_q, s_k, d, cls_n)
     stream = _current_stream(dev)
     if f16_only:
         # the caller only wants the fp16 result: the kernels' fp32 means go to the tail of the workspace
         # instead of a tensor of their own (one allocation less per call)
-        n_head = (n_ws + 255) & ~255
-        ws = _workspace(dev, stream, n_head + 4 * b * s_k)
+        ws = _workspace(dev, stream, n_ws + 4 * b * s_k)
         ws_ptr = ws.data_ptr()
-        out, out_ptr = None, ws_ptr + n_head
+        out, out_ptr = None, ws_ptr + n_ws
     else:
         out = torch.empty((b, s_k), dtype=torch.float32, device=dev)
         ws = _workspace(dev, stream, n_ws)
         ws_ptr, out_ptr = ws.data_ptr(), out.data_ptr()
     out_h = torch.empty((b, s_k), dtype=torch.float16, device=dev) if want_f16 else None
-    out_h_ptr = out_h.data_ptr() if want_f16 else None
-    qs, ks = _I64x4(*q.stride()), _I64x4(*k.stride())
-    bf16 = q.dtype == torch.bfloat16
-    cdll = _lib or lib()
-    if general:
-        rc = cdll.fcs_colsum_general(int(bf16), int(causal), q.data_ptr(), k.data_ptr(), out_ptr, out_h_ptr,
-                                     ws_ptr, n_ws, b, h, k.shape[1], s_q, s_k, d, int(cls_n), int(k_past),
-                                     qs, ks, scale, stream)
-        what = "fcs_colsum_general"
-    elif causal:
-        fn = cdll.fcs_colsum_causal_bf16 if bf16 else cdll.fcs_colsum_causal_f16
-        rc = fn(q.data_ptr(), k.data_ptr(), out_ptr, out_h_ptr, ws_ptr, n_ws, h, s_q, s_k, d, int(k_past), qs, ks, scale, stream)
-        what = "fcs_colsum_causal"
-    else:
-        fn = cdll.fcs_colsum_noncausal_bf16 if bf16 else cdll.fcs_colsum_noncausal_f16
-        rc = fn(q.data_ptr(), k.data_ptr(), out_ptr, out_h_ptr, ws_ptr, n_ws, b, h, s_q, d, qs, ks, scale, int(cls_n), stream)
-        what = "fcs_colsum_noncausal"
+    c.q, c.k, c.out, c.out_f16 = q.data_ptr(), k.data_ptr(), out_ptr, (out_h.data_ptr() if want_f16 else None)
+    c.ws, c.ws_bytes, c.hip_stream = ws_ptr, n_ws, stream
+    rc = (_lib or lib()).fcs_colsum_call(c_ref)
     if rc != 0:
-        _check(rc, what if general else what + ("_bf16" if bf16 else "_f16"))
+        _check(rc, "fcs_colsum_call")
     if f16_only:
         return out_h
     return (out, out_h) if want_f16 else out
 
 
 def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n: int, k_past: int, want_f16: bool = False,
-            general: bool = False, f16_only: bool = False):
+            f16_only: bool = False):
     """Enqueue one call; returns the fp32 means, (fp32, fp16) when `want_f16`, or the fp16 tensor alone
     when `f16_only` (which implies `want_f16`)."""
     want_f16 = want_f16 or f16_only
@@ -225,20 +270,39 @@ def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n:
         k = torch.nn.functional.pad(k.to(dtype), (0, pad))
     q = _as_kernel_input(q, dtype)
     k = _as_kernel_input(k, dtype)
+    # any k_past >= K_len means "no mask"; keep it inside the C int the library takes
+    k_past = min(int(k_past), k.shape[2])
     if q.device.index == torch.cuda.current_device():
-        return _enqueue(causal, q, k, float(scale), cls_n, k_past, want_f16, general, f16_only)
+        return _enqueue(causal, q, k, float(scale), cls_n, k_past, want_f16, f16_only)
     with torch.cuda.device(q.device):
-        return _enqueue(causal, q, k, float(scale), cls_n, k_past, want_f16, general, f16_only)
+        return _enqueue(causal, q, k, float(scale), cls_n, k_past, want_f16, f16_only)
+
+
+def plan_description(q_shape, k_shape, causal=False, cls_n=-1, k_past=None, scale=None, bf16=False) -> str:
+    """Text of the launch plan (kernels, template arguments, grids) a call of these dense shapes gets."""
+    b, h, s_q, d = q_shape
+    c = _Call()
+    c.struct_bytes = ctypes.sizeof(_Call)
+    c.dtype, c.causal = int(bf16), int(causal)
+    c.B, c.Hq, c.Hk, c.Sq, c.Sk, c.D = b, h, k_shape[1], s_q, k_shape[2], d
+    c.cls_n = -1 if cls_n is None or cls_n < 0 else int(cls_n)
+    c.k_past = (max(0, k_shape[2] - s_q) if k_past is None else min(int(k_past), k_shape[2])) if causal else 0
+    c.scale = float(d ** -0.5 if scale is None else scale)
+    c.q_strides = _I64x4(h * s_q * d, s_q * d, d, 1)
+    c.k_strides = _I64x4(k_shape[1] * k_shape[2] * d, k_shape[2] * d, d, 1)
+    buf = ctypes.create_string_buffer(1024)
+    lib().fcs_plan_describe(ctypes.byref(c), buf, len(buf))
+    return buf.value.decode()
 
 
 def colsum_general(Q: torch.Tensor, K: torch.Tensor, scale: float, causal: bool = False, CLS_N: int = -1,
                    K_past: Optional[int] = None, want_f16: bool = False):
-    """fcs_colsum_general: (B, S_k) fp32 means (or (fp32, fp16)) for grouped key heads, batched causal
-    calls, causal calls restricted to the first CLS_N rows and non-causal calls with S_q != S_k."""
+    """fcs_colsum_call in its general form: (B, S_k) fp32 means (or (fp32, fp16)) for grouped key heads,
+    batched causal calls, causal calls restricted to the first CLS_N rows and non-causal calls with S_q != S_k."""
     if K_past is None:
         K_past = max(0, K.shape[2] - Q.shape[2]) if causal else 0
-    return _launch(bool(causal), Q, K, scale, -1 if CLS_N is None or CLS_N < 0 else int(CLS_N), int(K_past), want_f16,
-                   general=True)
+    return _launch(bool(causal), Q, K, scale, -1 if CLS_N is None or CLS_N < 0 else int(CLS_N), int(K_past) if causal else 0,
+                   want_f16)
 
 
 def colsum_noncausal_f32(Q: torch.Tensor, K: torch.Tensor, scale: float, CLS_N: int = -1) -> torch.Tensor:

@@ -8,7 +8,7 @@
  * its three Triton launchers.  All pointers are DEVICE pointers unless stated otherwise.
  * The library never allocates, frees or synchronises: the caller owns the output and the
  * workspace, and every kernel is enqueued on the HIP stream passed in.  Calls are
- * re-entrant (no mutable global state).
+ * re-entrant (the only state kept between calls is a per-thread memo of recent launch plans).
  *
  * Return value of the launch functions: 0 = all kernels enqueued; negative = argument
  * error detected on the host before anything touched the GPU (FCS_E_*); positive = the
@@ -24,13 +24,13 @@
 extern "C" {
 #endif
 
-#define FCS_ABI_VERSION 4
+#define FCS_ABI_VERSION 5
 
 enum {
     FCS_OK = 0,
     FCS_E_NULL = -1,      /* a required pointer is NULL                                  */
-    FCS_E_DIMS = -2,      /* a dimension is < 1, or cls_n == 0, or k_past < 0, or B*H > 65535
-                             on the two-pass path (causal, S > 2048, S < 32 or D != 64)   */
+    FCS_E_DIMS = -2,      /* a dimension is < 1, or cls_n == 0, or k_past < 0, or the call
+                             would need 2^31 workgroups or more                          */
     FCS_E_HEAD_DIM = -3,  /* D is not a multiple of 8 in [8, 256]                        */
     FCS_E_STRIDE = -4,    /* last-dim stride != 1, or a stride / base not 16-B aligned   */
     FCS_E_WORKSPACE = -5, /* ws_bytes smaller than fcs_workspace_bytes() for these dims,
@@ -38,7 +38,8 @@ enum {
     FCS_E_SCALE = -6,     /* scale is NaN or infinite                                    */
     FCS_E_STATIC_LIMIT = -7, /* fcs_colsum_noncausal_f16_static: the call needs more workspace
                                 than FCS_STATIC_SCRATCH_BYTES                              */
-    FCS_E_DTYPE = -8      /* fcs_colsum_general: dtype is not FCS_DTYPE_F16 / FCS_DTYPE_BF16 */
+    FCS_E_DTYPE = -8,     /* fcs_colsum_general: dtype is not FCS_DTYPE_F16 / FCS_DTYPE_BF16 */
+    FCS_E_STRUCT = -9     /* fcs_colsum_call: struct_bytes is not sizeof(fcs_call_t)      */
 };
 
 /* Size of the per-GPU static scratch array behind fcs_colsum_noncausal_f16_static(). */
@@ -86,11 +87,17 @@ int fcs_colsum_noncausal_f16(const void *q, const void *k, float *out, void *out
  * fcs_workspace_bytes(0, B, H, S, S, D, cls_n) exceeds FCS_STATIC_SCRATCH_BYTES (8 MiB: enough
  * for B=8 H=16 S=2048 D=64, which needs 2 MiB).  All calls on one GPU share that GPU's array:
  * calls that overlap in time on one GPU (different streams or threads) race; calls on one
- * stream are ordered and safe.  Results are bit-identical to fcs_colsum_noncausal_f16. */
+ * stream are ordered and safe.  Results are bit-identical to fcs_colsum_noncausal_f16.
+ * The first call on a GPU looks up the array's device address (hipGetSymbolAddress), which may
+ * load the code object: make that call, or fcs_static_scratch_init(), outside stream capture.  A
+ * failed look-up is not remembered; the next call tries again. */
 int fcs_colsum_noncausal_f16_static(const void *q, const void *k, float *out, void *out_f16,
                                     int B, int H, int S, int D,
                                     const int64_t q_strides[4], const int64_t k_strides[4],
                                     float scale, int cls_n, void *hip_stream);
+
+/* Looks up the current GPU's static scratch array without launching anything (0, or a hipError_t). */
+int fcs_static_scratch_init(void);
 
 /* Causal column means for one sequence (batch 1), fp16 inputs, fp32 output.
  *   q          (1,H,Q_len,D), k (1,H,K_len,D) fp16; strides as above (index 0 ignored).
@@ -98,7 +105,8 @@ int fcs_colsum_noncausal_f16_static(const void *q, const void *k, float *out, vo
  *   out_f16    NULL, or (K_len) fp16 that additionally receives the rounded means.
  *   k_past     number of keys every query may see before its own position: key j is
  *              visible to query i  <=>  j <= k_past + i.  The reference infers
- *              max(0, K_len - Q_len); pass that for drop-in behaviour.
+ *              max(0, K_len - Q_len); pass that for drop-in behaviour.  Any value >= K_len
+ *              (INT_MAX included) means "no mask" and is treated as K_len.
  * Replaces `_flash_colsum_causal(Q, K, scale, K_past)` including its host epilogue
  * (reference: flash_colsum/kernel_causal.py:94-125; called from flash_colsum/ops.py:89). */
 int fcs_colsum_causal_f16(const void *q, const void *k, float *out, void *out_f16, void *ws, size_t ws_bytes,
@@ -142,6 +150,36 @@ int fcs_colsum_general(int dtype, int causal, const void *q, const void *k, floa
                        int cls_n, int k_past, const int64_t q_strides[4], const int64_t k_strides[4],
                        float scale, void *hip_stream);
 
+/* One call as a struct: the arguments of fcs_colsum_general().  For host layers whose
+ * foreign-function interface pays per argument (ctypes, cgo, JNI): fill the shape, strides and dtype
+ * once per tensor geometry, update the pointers and call.  The struct is only read.
+ *   struct_bytes  sizeof(fcs_call_t), checked (FCS_E_STRUCT).
+ *   flags         0 (reserved).
+ * All other fields mean what the like-named arguments of fcs_colsum_general() mean. */
+typedef struct fcs_call {
+    uint32_t struct_bytes;
+    uint32_t flags;
+    int32_t dtype, causal;
+    int32_t B, Hq, Hk, Sq, Sk, D;
+    int32_t cls_n, k_past;
+    float scale;
+    int32_t reserved;  /* 0 */
+    int64_t q_strides[4], k_strides[4];
+    const void *q, *k;
+    float *out;
+    void *out_f16;
+    void *ws;
+    size_t ws_bytes;
+    void *hip_stream;
+} fcs_call_t;
+int fcs_colsum_call(const fcs_call_t *call);
+
+/* Text description of the launch plan fcs_colsum_call() would use for `call` (kernels with their
+ * template arguments, grids, slabs), for benchmark records and logs; pointers in `call` are not
+ * dereferenced and may be NULL.  Writes at most buf_bytes - 1 characters plus a terminating NUL
+ * and returns the length of the full text (like snprintf); 0 for invalid dimensions. */
+size_t fcs_plan_describe(const fcs_call_t *call, char *buf, size_t buf_bytes);
+
 /* Selection over the fp32 means, for the consumer the reference names (token-importance ranking
  * for pruning, reference: README.md:10): it runs on the same stream right behind a launch function
  * above and reads its fp32 `out`, so the small means of long contexts are ranked before the fp16
@@ -157,6 +195,8 @@ int fcs_colsum_general(int dtype, int causal, const void *q, const void *k, floa
  * fcs_threshold_f32: for every row the positions of the entries >= tau, ascending.
  *   idx_out   (B,S) int64: row b holds count_out[b] positions (the rest is left untouched).
  *   count_out (B) int32.
+ *   `>=` is the comparison of values: -0 and +0 are equal, on either side.  (A NaN entry is listed
+ *   when its sign bit is clear and skipped when it is set; the means never hold one.)
  * Return codes as above (FCS_E_DIMS: k < 1, k > S, or sorted with k > FCS_TOPK_SORT_MAX;
  * FCS_E_SCALE: tau is NaN). */
 #define FCS_TOPK_SORT_MAX 4096

@@ -495,11 +495,78 @@ def test_captured_call_owns_its_workspace():
         del junk
 
 
-def test_explicit_k_past():
-    """The causal launcher's K_past argument (reference: kernel_causal.py:94-113)."""
+def test_struct_call_gives_the_bits_of_the_argument_list_entry_points():
+    """fcs_colsum_call (one struct) against fcs_colsum_noncausal_f16 / fcs_colsum_causal_f16 (argument lists):
+    the same plan, the same kernels, the same bits; the struct is reused across calls with new pointers."""
     from flash_colsum import _hip
 
+    lib = _hip.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    for qs, ks, causal, cls_n in [((3, 5, 333, 64), (3, 5, 333, 64), False, -1), ((4, 6, 577, 64), (4, 6, 577, 64), False, 1),
+                                  ((1, 4, 96, 128), (1, 4, 3000, 128), True, -1), ((2, 4, 512, 64), (2, 4, 512, 64), False, -1)]:
+        q, k = _inputs(qs, ks, seed=41)
+        q, k = q.cuda(), k.cuda()
+        b, h, sq, d = qs
+        sk = ks[2]
+        k_past = max(0, sk - sq) if causal else 0
+        c, c_ref, n_ws = _hip._prepared_call(causal, q, k, 0.125, cls_n, k_past)
+        assert n_ws == lib.fcs_workspace_bytes(int(causal), b, h, sq, sk, d, cls_n)
+        ws = torch.full((max(n_ws, 1),), 0xA5, dtype=torch.uint8, device="cuda")
+        st = (ctypes.c_int64 * 4)(*q.stride()), (ctypes.c_int64 * 4)(*k.stride())
+        want = torch.full((b, sk), float("nan"), dtype=torch.float32, device="cuda")
+        if causal:
+            rc = lib.fcs_colsum_causal_f16(q.data_ptr(), k.data_ptr(), want.data_ptr(), None, ws.data_ptr(), n_ws, h, sq, sk, d,
+                                           k_past, st[0], st[1], 0.125, stream)
+        else:
+            rc = lib.fcs_colsum_noncausal_f16(q.data_ptr(), k.data_ptr(), want.data_ptr(), None, ws.data_ptr(), n_ws, b, h, sq, d,
+                                              st[0], st[1], 0.125, cls_n, stream)
+        assert rc == 0
+        for rep in range(2):
+            out = torch.full((b, sk), float("nan"), dtype=torch.float32, device="cuda")
+            out_h = torch.full((b, sk), float("nan"), dtype=torch.float16, device="cuda")
+            c.q, c.k, c.out, c.out_f16 = q.data_ptr(), k.data_ptr(), out.data_ptr(), out_h.data_ptr()
+            c.ws, c.ws_bytes, c.hip_stream = ws.data_ptr(), n_ws, stream
+            assert lib.fcs_colsum_call(c_ref) == 0
+            torch.cuda.synchronize()
+            assert torch.equal(out, want) and torch.equal(out_h, want.half()), (qs, rep)
+
+
+def test_more_than_65535_batch_entries_times_heads():
+    """The two-pass kernels take (batch entry, head) on a one-dimensional grid: B * H is not limited to 16 bits.
+    Batch entries are independent, so a few of them (first, last, either side of 65536 / H) are checked against
+    the oracle and all of them through the row sums of the means."""
+    for shape, what in [((4100, 16, 8, 128), "B*H = 65600, two-pass path"), ((1100, 64, 40, 64), "B*H = 70400, fused path")]:
+        q, k = _inputs(shape, shape, seed=43)
+        out = _run(q, k)
+        pick = torch.tensor([0, 1, shape[0] // 2, 65536 // shape[1] - 1, 65536 // shape[1], shape[0] - 2, shape[0] - 1])
+        _assert_close(out.cpu()[pick], _oracle(q[pick], k[pick]), what)
+        assert (out.double().sum(-1) - 1.0).abs().max().item() < 1e-5, what
+
+
+def test_explicit_k_past():
+    """The causal launcher's K_past argument (reference: kernel_causal.py:94-113).  Every k_past >= K_len - 1
+    means "no mask": 199, 500 and the largest C int give the bits of the unmasked call."""
+    from flash_colsum import _hip, flash_colsum_ext
+
     q, k = _inputs((1, 3, 40, 64), (1, 3, 200, 64), seed=4)
+    unmasked = _hip.colsum_general(q.cuda(), k.cuda(), 0.125, causal=True, K_past=199)
+    for k_past in (200, 2 ** 31 - 1, 2 ** 40):
+        assert torch.equal(_hip.colsum_causal_f32(q.cuda(), k.cuda(), 0.125, K_past=k_past), unmasked), k_past
+        assert torch.equal(flash_colsum_ext(q.cuda(), k.cuda(), 0.125, is_causal=True, k_past=k_past, out_dtype=torch.float32),
+                           unmasked), k_past
+    p = torch.softmax((q.double() @ k.double().transpose(-1, -2)) * 0.125, -1)
+    _assert_close(unmasked, p.mean((1, 2)), "k_past >= K_len - 1")
+    # the same through the raw C entry point with INT_MAX
+    lib = _hip.lib()
+    qc, kc = q.cuda(), k.cuda()
+    n_ws = lib.fcs_workspace_bytes(1, 1, 3, 40, 200, 64, -1)
+    ws = torch.empty(n_ws, dtype=torch.uint8, device="cuda")
+    out = torch.full((1, 200), float("nan"), dtype=torch.float32, device="cuda")
+    st = (ctypes.c_int64 * 4)(*qc.stride()), (ctypes.c_int64 * 4)(*kc.stride())
+    rc = lib.fcs_colsum_causal_f16(qc.data_ptr(), kc.data_ptr(), out.data_ptr(), None, ws.data_ptr(), n_ws, 3, 40, 200, 64,
+                                   2 ** 31 - 1, st[0], st[1], 0.125, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0 and torch.equal(out, unmasked)
     for k_past in (0, 37, 160, 199, 500):
         out = _hip.colsum_causal_f32(q.cuda(), k.cuda(), 0.125, K_past=k_past)
         s = (q.double() @ k.double().transpose(-1, -2)) * 0.125
@@ -698,13 +765,31 @@ def test_threshold_kernel_bit_exact():
     g = torch.Generator().manual_seed(3)
     x = torch.rand((3, 4097), generator=g, dtype=torch.float32)
     x[:, ::5] = 0.25
-    for tau in (0.25, 0.0, 0.999, 2.0, -1.0):
+    x[:, 7::11] = 0.0
+    x[:, 3::13] = -0.0  # equal to +0 under >=, whichever side carries the sign
+    x[:, 1::17] = -0.5
+    for tau in (0.25, 0.0, -0.0, 0.999, 2.0, -1.0, -0.5):
         idx, cnt = _hip.threshold_f32(x.cuda(), tau)
         torch.cuda.synchronize()
         for r in range(3):
             want = (x[r] >= tau).nonzero().view(-1)
             assert cnt[r].item() == want.numel(), (tau, r)
             assert torch.equal(idx[r, : want.numel()].cpu(), want)
+
+
+def test_topk_sorts_padding_behind_every_real_entry():
+    """k below the next power of two: the sorting network's padding must not displace real entries, whatever
+    their sign (the column means are never negative; the kernel takes any floats)."""
+    from flash_colsum import _hip
+
+    g = torch.Generator().manual_seed(8)
+    x = -torch.rand((2, 300), generator=g, dtype=torch.float32) * 1e30
+    x[0, 5] = float("-inf")
+    for k in (5, 37, 300):
+        val, idx = _hip.topk_f32(x.cuda(), k, sorted=True)
+        torch.cuda.synchronize()
+        want = torch.sort(x, dim=1, descending=True, stable=True)
+        assert torch.equal(val.cpu(), want.values[:, :k]) and torch.equal(idx.cpu(), want.indices[:, :k]), k
 
 
 @pytest.mark.parametrize("qs,ks,kw,k", [

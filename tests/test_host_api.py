@@ -63,14 +63,15 @@ def test_library_exports_every_declared_symbol():
     names = _declared_symbols()
     assert set(names) >= {"fcs_abi_version", "fcs_colsum_causal_bf16", "fcs_colsum_causal_f16", "fcs_colsum_noncausal_bf16",
                           "fcs_colsum_noncausal_f16", "fcs_colsum_noncausal_f16_static", "fcs_colsum_general",
-                          "fcs_topk_f32", "fcs_threshold_f32", "fcs_strerror", "fcs_workspace_bytes"}
+                          "fcs_topk_f32", "fcs_threshold_f32", "fcs_strerror", "fcs_workspace_bytes", "fcs_colsum_call",
+                          "fcs_plan_describe", "fcs_static_scratch_init"}
     for n in names:
         assert getattr(lib, n) is not None
-    assert lib.fcs_abi_version() == 4
+    assert lib.fcs_abi_version() == 5
 
 
 def test_strerror_is_total():
-    for code in range(-8, 3):
+    for code in range(-9, 3):
         assert isinstance(_hip.strerror(code), str) and _hip.strerror(code)
     assert "head dim" in _hip.strerror(-3)
 
@@ -147,6 +148,97 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert nb(p, p, p, None, p, 16, 2, 8, 16, 64, st, st, 0.125, -1, None) == -5
     assert cb(p, p, p, None, p, 1 << 30, 8, 16, 64, 64, -1, st, st, 0.125, None) == -2
     assert cb(p, p, p, None, p, 16, 8, 16, 64, 64, 48, st, st, 0.125, None) == -5
+
+
+def _call_struct(**kw):
+    c = _hip._Call()
+    c.struct_bytes = ctypes.sizeof(_hip._Call)
+    c.dtype, c.causal, c.B, c.Hq, c.Hk, c.Sq, c.Sk, c.D, c.cls_n, c.k_past, c.scale = 0, 0, 2, 8, 8, 16, 16, 64, -1, 0, 0.125
+    c.q_strides = (ctypes.c_int64 * 4)(8 * 16 * 64, 16 * 64, 64, 1)
+    c.k_strides = (ctypes.c_int64 * 4)(8 * 16 * 64, 16 * 64, 64, 1)
+    c.q = c.k = c.out = c.ws = 4096  # never dereferenced
+    c.ws_bytes = 1 << 30
+    for name, v in kw.items():
+        setattr(c, name, v)
+    return c
+
+
+def test_struct_call_reports_argument_errors_without_a_gpu():
+    lib = _hip.lib()
+    call = lib.fcs_colsum_call
+    assert call(None) == -1
+    assert call(ctypes.byref(_call_struct(struct_bytes=8))) == -9 and "fcs_call_t" in _hip.strerror(-9)
+    assert call(ctypes.byref(_call_struct(dtype=7))) == -8
+    assert call(ctypes.byref(_call_struct(q=None))) == -1
+    assert call(ctypes.byref(_call_struct(B=0))) == -2
+    assert call(ctypes.byref(_call_struct(Hk=3))) == -2
+    assert call(ctypes.byref(_call_struct(causal=1, k_past=-1))) == -2
+    assert call(ctypes.byref(_call_struct(D=12))) == -3
+    assert call(ctypes.byref(_call_struct(q=4098))) == -4
+    assert call(ctypes.byref(_call_struct(ws_bytes=1024))) == -5
+    assert call(ctypes.byref(_call_struct(ws=4100))) == -5
+    assert call(ctypes.byref(_call_struct(scale=float("inf")))) == -6
+    # the struct mirrors the C declaration field for field
+    text = open(os.path.join(ROOT, "include", "flash_colsum.h")).read()
+    body = re.search(r"typedef struct fcs_call \{(.*?)\} fcs_call_t;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    declared = []
+    for stmt in body.split(";"):
+        stmt = stmt.strip()
+        if stmt:
+            declared += [n.strip(" *").split("[")[0] for n in stmt.split(",")]
+            declared[-len(stmt.split(",")):] = [n.split()[-1].strip("*") for n in declared[-len(stmt.split(",")):]]
+    assert declared == [f[0] for f in _hip._Call._fields_], declared
+
+
+def test_plan_description_and_k_past_clamp():
+    """The launch plan as text: which kernels a call gets.  Any k_past >= K_len means "no mask" and must plan
+    (and run) like k_past = K_len, INT_MAX included: the kernels add it to row numbers in 32 bits."""
+    d = _hip.plan_description
+    t = d((8, 16, 2048, 64), (8, 16, 2048, 64))
+    assert "fcs_fused_kernel<64,8,false,8,false,true>" in t and "fcs_finalize_kernel<8>" in t
+    assert "fcs_fewrows_kernel<64,1,false>" in d((32, 16, 577, 64), (32, 16, 577, 64), cls_n=1)
+    t = d((1, 32, 512, 128), (1, 32, 65536, 128), causal=True)
+    assert "fcs_rowstream_kernel<128,2,8,false,false>" in t and "fcs_colstream_kernel<128,2,8,false,false>" in t
+    assert "bf16" not in t and "fcs_fused_kernel<64,8,true,8,true,false>" in d((8, 16, 2048, 64), (8, 16, 2048, 64), bf16=True)
+    base = d((1, 4, 100, 128), (1, 4, 1000, 128), causal=True, k_past=1000)
+    for kp in (1001, 5000, 2 ** 31 - 1, 2 ** 40):
+        assert d((1, 4, 100, 128), (1, 4, 1000, 128), causal=True, k_past=kp) == base
+    c = _call_struct(causal=1, Sq=100, Sk=1000, k_past=2 ** 31 - 1)
+    buf = ctypes.create_string_buffer(1024)
+    n = _hip.lib().fcs_plan_describe(ctypes.byref(c), buf, len(buf))
+    c.k_past = 1000
+    buf2 = ctypes.create_string_buffer(1024)
+    assert n > 0 and _hip.lib().fcs_plan_describe(ctypes.byref(c), buf2, len(buf2)) == n and buf.value == buf2.value
+    # snprintf semantics: truncated output, full length returned
+    small = ctypes.create_string_buffer(8)
+    assert _hip.lib().fcs_plan_describe(ctypes.byref(c), small, len(small)) == n and len(small.value) == 7
+    assert _hip.lib().fcs_plan_describe(ctypes.byref(_call_struct(B=0)), buf, len(buf)) == 0
+
+
+def test_more_than_65535_batch_entries_times_heads_plan():
+    """Both passes of the two-pass path launch one-dimensional grids: no 16-bit grid axis limits B * H."""
+    assert _hip.workspace_bytes(False, 4096, 32, 64, 4096, 64) > 0
+    assert _hip.workspace_bytes(True, 70000, 1, 8, 300, 128) > 0
+    assert "grid" in _hip.plan_description((4096, 32, 64, 128), (4096, 32, 64, 128))
+
+
+def test_kernel_inputs_with_odd_strides_on_unit_dimensions():
+    """torch calls a tensor contiguous whatever the strides of its size-1 dimensions; the library wants every
+    stride a multiple of 8 elements, so such tensors must still be checked (and copied when needed)."""
+    import torch
+
+    base = torch.zeros(4 * 77 * 64 + 64, dtype=torch.float16)
+    t = base.as_strided((4, 1, 77, 64), (77 * 64, 3, 64, 1))  # one head, head stride 3
+    assert t.is_contiguous()
+    u = _hip._as_kernel_input(t)
+    assert u.stride(1) % 8 == 0 and u.stride(2) % 8 == 0
+    t = base.as_strided((4, 2, 1, 64), (2 * 64, 64, 5, 1))  # one row, row stride 5
+    assert t.is_contiguous()
+    u = _hip._as_kernel_input(t)
+    assert u.stride(1) % 8 == 0 and u.stride(2) % 8 == 0
+    v = torch.zeros((2, 3, 16, 64), dtype=torch.float16)
+    assert _hip._as_kernel_input(v) is v
 
 
 def test_topk_argument_errors_without_a_gpu():

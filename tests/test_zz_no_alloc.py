@@ -38,13 +38,20 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
     # a ragged fused call, a two-pass call (row statistics + partials) and a few-rows call
     cases = [((8, 16, 2048, 64), -1, 0.125), ((3, 5, 333, 64), -1, 0.2), ((2, 3, 300, 128), -1, 0.1),
              ((4, 6, 577, 64), 1, 0.125), ((1, 2, 40, 64), -1, 0.125)]
+    assert lib.fcs_static_scratch_init() == 0  # the look-up of the array's address, outside any capture
     for shape, cls_n, scale in cases:
         q = torch.randn(shape, generator=g).half()
         k = torch.randn(shape, generator=g).half()
         qc, kc = q.cuda(), k.cuda()
         print("static entry point", shape, cls_n, flush=True)
         rc0, want, want_h = _call(lib, False, qc, kc, cls_n, scale)
+        # the static call itself allocates nothing: device memory in use is the same before and after it,
+        # the output tensors of _call() aside (they come out of torch's cache, which the warm-up call filled)
+        _call(lib, True, qc, kc, cls_n, scale)
+        free0, _ = torch.cuda.mem_get_info()
         rc1, got, got_h = _call(lib, True, qc, kc, cls_n, scale)
+        free1, _ = torch.cuda.mem_get_info()
+        assert free1 == free0, (shape, free0, free1)
         assert rc0 == 0 and rc1 == 0, (shape, rc0, rc1)
         assert torch.equal(got, want) and torch.equal(got_h, want_h), shape
         ref = colsum_exact(q, k, scale=scale, cls_len=None if cls_n < 0 else cls_n)
