@@ -121,6 +121,8 @@ int prepare(fcs::Plan &p, fcs::Args &a, int bf16, int causal, const void *q, con
     a.kv_magic = (uint32_t)((0x100000000ull + (uint64_t)a.kv_group - 1) / (uint64_t)a.kv_group);  // unused when the group is 1
     a.q_rows = p.q_rows;
     a.causal = p.causal; a.k_past = p.k_past;
+    // keys j <= k_past are visible to every row; whole stages of them
+    a.pre_end = p.causal ? (int)((((long)p.k_past + 1) / fcs::kStageKeys) * fcs::kStageKeys) : 0x3fffffc0;
     a.negate = scale < 0.f;
     a.c = fabsf(scale) * 1.44269504088896340736f;
     a.n_chunks = p.n_chunks; a.chunk_keys = p.chunk_keys; a.rows_pad = p.rows_pad;

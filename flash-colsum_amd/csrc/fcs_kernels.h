@@ -18,6 +18,8 @@ struct Args {
     uint32_t kv_magic;   // ceil(2^32 / kv_group), for the division above (unused when kv_group == 1)
     int q_rows;          // query rows that are averaged
     int causal, k_past;  // key j visible to query i  <=>  j <= k_past + i
+    int pre_end;         // two-pass path, pre-scaled variant: the 64-key stages that end at or below this key (a multiple
+                         // of 64) run on Q * c rounded to fp16 in both passes; the keys that every averaged row sees
     int negate;          // scale < 0: scores are negated by flipping the stationary operand's sign
     float c;             // |scale| * log2(e)
     // pass 1

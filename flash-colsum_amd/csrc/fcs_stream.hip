@@ -91,10 +91,14 @@ __device__ __forceinline__ half8 prescale(half8 v, float cs)
 
 }  // namespace
 
-// PRE (fp16, D = 64, non-causal only; chosen by the launcher when at least 16384 (head, row) pairs are
-// averaged and |scale| <= 1/8): the stationary operand is Q * c rounded to fp16, the row constant is -log2 l_i, and
-// p_ij = 2^(s'_ij - log2 l_i) costs a v_exp_f32 alone.  Pass 1 made l_i from the same pre-scaled scores.
-// Units with a stabilised row keep the raw operand and the two-constant form.
+// PRE (fp16, D = 64; chosen by the launcher when at least 16384 (head, row) pairs are averaged and
+// |scale| <= 1/8): for the keys below a.pre_end the stationary operand is Q * c rounded to fp16, the row constant
+// is -log2 l_i, and p_ij = 2^(s'_ij - log2 l_i) costs a v_exp_f32 alone.  Pass 1 made l_i from the same scores:
+// both passes decide per 64-key stage, by the stage's position alone (stages that end at or below a.pre_end, a
+// multiple of 64: every key of a non-causal call; the keys that EVERY row sees of a causal one, whose last keys
+// are averaged over few rows and keep the raw operand).  A unit therefore streams in up to two phases, the
+// pre-scaled stages first, then the raw ones after reloading Q.  Units with a stabilised row keep the raw operand
+// and the two-constant form throughout.
 template <int D, int NB, int WAVES, bool BF, bool PRE>
 __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args a)
 {
@@ -115,7 +119,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
     static_assert(NS >= 3, "the ring holds the stage in use, the next one and at least one in flight");
     __shared__ __attribute__((aligned(16))) char ring[NS * STAGE_BYTES];
     __shared__ __attribute__((aligned(16))) float colw[WAVES * CHUNK];  // per-wave column sums of the chunk
-    __shared__ __attribute__((aligned(16))) float nl_s[BLOCK_ROWS];     // per-row constants of the current unit
+    __shared__ __attribute__((aligned(16))) float nl_s[BLOCK_ROWS];     // per-row constants of the current unit: -log2(l_i) / c
+    __shared__ __attribute__((aligned(16))) float np_s[PRE ? BLOCK_ROWS : 4];  // the same for pre-scaled scores: -log2(l_i)
     __shared__ __attribute__((aligned(16))) float lg_s[BLOCK_ROWS];     // log2 l_i, used by units with stabilised rows
     __shared__ __attribute__((aligned(16))) float cm_s[BLOCK_ROWS];     // -m_i of those units
     __shared__ int shift_s[WAVES];                                       // per wave: one of its rows is stabilised
@@ -195,36 +200,50 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
                     }
                     lg = fast_log2(ll);
                 }
-                nl = (PRE || a.c == 0.f) ? -lg : -lg / a.c;
+                nl = (a.c == 0.f) ? -lg : -lg / a.c;
             }
             // a stabilised row anywhere in the unit switches the whole unit to the two-constant form
             const bool sh = __builtin_amdgcn_ballot_w64(mm != 0.f) != 0;
             if (lane == 0) shift_s[wave] = sh ? 1 : 0;
             if (tid < BLOCK_ROWS) {
                 nl_s[tid] = nl;
+                if (PRE) np_s[tid] = (nl == -INFINITY) ? -INFINITY : -lg;
                 lg_s[tid] = lg;
                 cm_s[tid] = (nl == -INFINITY) ? -INFINITY : -mm;
             }
         }
 
-        // ---- stationary operand: this wave's query rows of head h
+        // ---- stationary operand: this wave's query rows of head h, as they are in memory
         const int qw0 = row0 + wave * ROWS_W;
         half8 qf[NB][NT];
-        {
+        auto load_q_rows = [&]() {
             const _Float16 *qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h;
+            int lane_o = lane;
+            asm volatile("" : "+v"(lane_o));  // addresses are formed here, not kept for a second call
+            const int n_o = lane_o & 31, g_o = lane_o >> 5;
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-                const _Float16 *row = qp + (int64_t)min(qw0 + nb * 32 + n, a.Sq - 1) * a.qs_s + g * 8;
+                const _Float16 *row = qp + (int64_t)min(qw0 + nb * 32 + n_o, a.Sq - 1) * a.qs_s + g_o * 8;
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
                     half8 v = kZero8;  // channels past the tensor's head dim are zeros
-                    if (t * 16 + g * 8 < a.D) v = load8(row + t * 16);
-                    if (!PRE && a.negate) v = flip_sign(v);
+                    if (t * 16 + g_o * 8 < a.D) v = load8(row + t * 16);
                     if (a.c == 0.f) v = kZero8;
                     qf[nb][t] = v;
                 }
             }
-        }
+        };
+        // the form the matrix pipe takes: pre-scaled (sign included), or raw with the scale's sign
+        auto shape_q = [&](bool scaled) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    if (PRE && scaled) qf[nb][t] = prescale(qf[nb][t], a.negate ? -a.c : a.c);
+                    else if (a.negate) qf[nb][t] = flip_sign(qf[nb][t]);
+                }
+        };
+        load_q_rows();
         const char *kp = reinterpret_cast<const char *>(a.k + (int64_t)b * a.ks_b +
                                                         (int64_t)kv_head(h, a.kv_group, a.kv_magic) * a.ks_h);
         const int64_t k_row_b = a.ks_s * 2;
@@ -278,7 +297,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
             }
         };
 
-        // ---- prologue: NS - 1 stages in flight; stages 0 and 1 must have landed before the first barrier
+        // ---- prologue of the unit's first phase: NS - 1 stages in flight; stages 0 and 1 must have landed
+        // before the first barrier
 #pragma unroll
         for (int st = 0; st < NS - 1; ++st) fetch_stage(st, st);
         FCS_WAIT_VM((NS - 3) * IPW);
@@ -291,179 +311,197 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
             asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(f) : "v"(ad) : "memory");
             shifted = __builtin_amdgcn_ballot_w64(f != 0) != 0;
         }
-        if (PRE) {  // block-uniform choice: scaled operand, or the raw one (with the scale's sign) for the two-constant form
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    if (!shifted) qf[nb][t] = prescale(qf[nb][t], a.negate ? -a.c : a.c);
-                    else if (a.negate) qf[nb][t] = flip_sign(qf[nb][t]);
-                }
-        }
-        floatx16 cinit[NB];  // row constants in accumulator layout: register i <-> row 8*(i/4) + 4*g + i%4
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-                floatx4 v;  // inline assembly for the same reason as the operand reads below
-                const uint32_t ad = lds_addr(nl_s) + (uint32_t)((wave * ROWS_W + nb * 32 + 8 * i4 + 4 * g) * 4);
-                asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(ad) : "memory");
-#pragma unroll
-                for (int j = 0; j < 4; ++j) cinit[nb][4 * i4 + j] = shifted ? 0.f : v[j];
-            }
+        // leading stages of the unit that run on the pre-scaled operand (block-uniform)
+        const int n_pre = (!PRE || shifted) ? 0 : min(nst, max(0, (a.pre_end - c0) / KT));
 
         // rows of this wave relative to the causal diagonal; non-causal: every key below Sk is visible
         const int kp_eff = a.causal ? a.k_past : 0x3fffffff - a.Sq;
         const int thr_wave_min = a.causal ? min(a.k_past + qw0, a.Sk - 1) : a.Sk - 1;   // last key EVERY row of the wave sees
 
-        // ---- the stream.  A stage is NA * NB tiles of 32 rows x 32 keys; tile q = na * NB + nb uses key
-        // fragment na and accumulator q & 1.  Software pipeline inside the wave: the MFMA chain of tile q
-        // is issued BEFORE the exponent work of tile q - 1, so the matrix pipe and the VALU run together
-        // whatever the phase of the other wave on the SIMD.
-        constexpr int TILES = NA * NB;
-        static_assert(TILES % 2 == 0, "two accumulators alternate");
-        half8 kf[NT];
-        take_frag(std::integral_constant<int, 0>{}, kf);
-        floatx16 acc[2];
+        // One phase: the stages [s0, s1) of the unit in one form of the operand (SC: pre-scaled).  `fetched`: the
+        // phase's first NS - 1 stages are already in the ring (the unit's prologue above).
+        auto run_phase = [&](auto sc_c, const int s0, const int s1, const bool fetched) {
+            constexpr bool SC = decltype(sc_c)::value;
+            if (!fetched) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[0][i] = acc[1][i] = 0.f;
-        float cp[4] = {0.f, 0.f, 0.f, 0.f};  // running column sums of the fragment being exponentiated
-
-        // Exponent work of one finished tile (kb_t: first key of its stage), split in three so that the
-        // common case can be woven between the MFMAs of the next tile:
-        //   drain_begin   requests the fragment's accumulator slot (first row fragment only)
-        //   drain_slow    masked / stabilised forms, all sixteen scores at once
-        //   drain_end     after the last row fragment: fold the half-waves, add into the wave's slice
-        float col_old = 0.f;
-        uint32_t col_ad = 0;
-        auto drain_begin = [&](int kb_t, int na, int nb) {
-            if (nb == 0) {
-                col_ad = lds_addr(colw_w) + (uint32_t)((kb_t - c0 + na * 32 + n) * 4);
-                asm volatile("ds_read_b32 %0, %1" : "=v"(col_old) : "v"(col_ad) : "memory");
+                for (int st = 0; st < NS - 1; ++st) fetch_stage(s0 + st, st);
+                FCS_WAIT_VM((NS - 3) * IPW);
+                block_sync();
             }
-        };
-        auto drain_slow = [&](const floatx16 &sc, int kb_t, int na, int nb) {
-            const int key = kb_t + na * 32 + n;
-            // visible  <=>  key < Sk  and  key - k_past - (row of register i) <= 0
-            int rel = (key < a.Sk) ? key - kp_eff - (qw0 + 4 * g) : 0x3fffffff;
-            asm volatile("" : "+v"(rel));
-            if (shifted) {
-                // rare: the accumulators started at 0, so the scores carry the very bits pass 1 saw;
-                // m_i is subtracted before the scale and log2 l_i after it
+            floatx16 cinit[NB];  // row constants in accumulator layout: register i <-> row 8*(i/4) + 4*g + i%4
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
-                    floatx4 l4, m4;
-                    const uint32_t ro = (uint32_t)((wave * ROWS_W + nb * 32 + 8 * i4 + 4 * g) * 4);
-                    const uint32_t ad = lds_addr(lg_s) + ro, am = lds_addr(cm_s) + ro;
-                    asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
-                                 : "=&v"(l4), "=&v"(m4)
-                                 : "v"(ad), "v"(am)
-                                 : "memory");
+                    floatx4 v;  // inline assembly for the same reason as the operand reads
+                    const uint32_t ad = lds_addr(SC ? np_s : nl_s) + (uint32_t)((wave * ROWS_W + nb * 32 + 8 * i4 + 4 * g) * 4);
+                    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(ad) : "memory");
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float pr = fast_exp2(fmaf(sc[4 * i4 + j] + m4[j], cmul, -l4[j]));
-                        cp[j] += (rel <= nb * 32 + 8 * i4 + j) ? pr : 0.f;
+                    for (int j = 0; j < 4; ++j) cinit[nb][4 * i4 + j] = shifted ? 0.f : v[j];
+                }
+
+            // ---- the stream.  A stage is NA * NB tiles of 32 rows x 32 keys; tile q = na * NB + nb uses key
+            // fragment na and accumulator q & 1.  Software pipeline inside the wave: the MFMA chain of tile q
+            // is issued BEFORE the exponent work of tile q - 1, so the matrix pipe and the VALU run together
+            // whatever the phase of the other wave on the SIMD.
+            constexpr int TILES = NA * NB;
+            static_assert(TILES % 2 == 0, "two accumulators alternate");
+            half8 kf[NT];
+            take_frag(std::integral_constant<int, 0>{}, kf);
+            floatx16 acc[2];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[0][i] = acc[1][i] = 0.f;
+            float cp[4] = {0.f, 0.f, 0.f, 0.f};  // running column sums of the fragment being exponentiated
+
+            // Exponent work of one finished tile (kb_t: first key of its stage), split in three so that the
+            // common case can be woven between the MFMAs of the next tile:
+            //   drain_begin   requests the fragment's accumulator slot (first row fragment only)
+            //   drain_slow    masked / stabilised forms, all sixteen scores at once
+            //   drain_end     after the last row fragment: fold the half-waves, add into the wave's slice
+            float col_old = 0.f;
+            uint32_t col_ad = 0;
+            auto drain_begin = [&](int kb_t, int na, int nb) {
+                if (nb == 0) {
+                    col_ad = lds_addr(colw_w) + (uint32_t)((kb_t - c0 + na * 32 + n) * 4);
+                    asm volatile("ds_read_b32 %0, %1" : "=v"(col_old) : "v"(col_ad) : "memory");
+                }
+            };
+            auto drain_slow = [&](const floatx16 &sc, int kb_t, int na, int nb) {
+                const int key = kb_t + na * 32 + n;
+                // visible  <=>  key < Sk  and  key - k_past - (row of register i) <= 0
+                int rel = (key < a.Sk) ? key - kp_eff - (qw0 + 4 * g) : 0x3fffffff;
+                asm volatile("" : "+v"(rel));
+                if (shifted) {
+                    // rare: the accumulators started at 0, so the scores carry the very bits pass 1 saw;
+                    // m_i is subtracted before the scale and log2 l_i after it
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) {
+                        floatx4 l4, m4;
+                        const uint32_t ro = (uint32_t)((wave * ROWS_W + nb * 32 + 8 * i4 + 4 * g) * 4);
+                        const uint32_t ad = lds_addr(lg_s) + ro, am = lds_addr(cm_s) + ro;
+                        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
+                                     : "=&v"(l4), "=&v"(m4)
+                                     : "v"(ad), "v"(am)
+                                     : "memory");
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const float pr = fast_exp2(fmaf(sc[4 * i4 + j] + m4[j], cmul, -l4[j]));
+                            cp[j] += (rel <= nb * 32 + 8 * i4 + j) ? pr : 0.f;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const float pr = fast_exp2(SC ? sc[i] : sc[i] * cmul);
+                        cp[i & 3] += (rel <= nb * 32 + 8 * (i >> 2) + (i & 3)) ? pr : 0.f;
                     }
                 }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float pr = fast_exp2(PRE ? sc[i] : sc[i] * cmul);
-                    cp[i & 3] += (rel <= nb * 32 + 8 * (i >> 2) + (i & 3)) ? pr : 0.f;
+            };
+            auto drain_end = [&](int nb) {
+                if (nb == NB - 1) {
+                    float tot = (cp[0] + cp[1]) + (cp[2] + cp[3]);
+                    cp[0] = cp[1] = cp[2] = cp[3] = 0.f;
+                    // v_permlane32_swap exchanges the upper half of its first operand with the lower half of
+                    // its second: started from two copies of the value, one register then holds the lower
+                    // half-wave's values in both halves and the other the upper half-wave's, so their sum is
+                    // the total of the two half-waves in every lane.  (Inline assembly: given the same value
+                    // twice, the builtin's two results were folded into one.)
+                    float x = tot, y = tot;
+                    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
+                    tot = x + y;
+                    // plain read-modify-write of the wave's own slot (LDS float atomics are slow): the old
+                    // value was requested before the exponent work; both half-waves store the same total
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(col_old)::"memory");
+                    tot += col_old;
+                    asm volatile("ds_write_b32 %0, %1" ::"v"(col_ad), "v"(tot) : "memory");
                 }
+            };
+
+            // MFMA chain of one tile alone
+            auto chain = [&](int nb) {
+                floatx16 c = mfma16<BF>(qf[nb][0], kf[0], cinit[nb]);
+#pragma unroll
+                for (int t = 1; t < NT; ++t) c = mfma16<BF>(qf[nb][t], kf[t], c);
+                return c;
+            };
+            auto drain_fast = [&](const floatx16 &sc) {  // every key of the tile visible, no stabilised row
+#pragma unroll
+                for (int i = 0; i < 16; ++i) cp[i & 3] += fast_exp2(SC ? sc[i] : sc[i] * cmul);
+            };
+
+            // one stage, in ring slot SLOT (compile-time)
+            auto stage = [&](int st, auto slot_c) {
+                constexpr int SLOT = decltype(slot_c)::value;
+                const int kb = c0 + st * KT;
+                if (st > s0) {
+                    // stage st + 1 has landed (this wave's pieces; the barrier extends that to everyone's), and
+                    // every wave is done reading stage st - 1, whose slot takes the next fetch
+                    FCS_WAIT_VM((NS - 3) * IPW);
+                    block_barrier();
+                }
+                fetch_stage(st + NS - 1, (SLOT + NS - 1) % NS);
+#pragma unroll
+                for (int q = 0; q < TILES; ++q) {
+                    const int na = q / NB, nb = q % NB;
+                    // the previous tile: the one before in this stage, or the last of the previous stage
+                    const int p_kb = (q > 0) ? kb : kb - KT;
+                    const int p_na = (q > 0) ? (q - 1) / NB : NA - 1, p_nb = (q > 0) ? (q - 1) % NB : NB - 1;
+                    const bool have_prev = (q > 0) || (st > s0);
+                    const bool p_fast = !shifted && !(p_kb + p_na * 32 + 31 > thr_wave_min);  // wave-uniform
+                    auto do_chain = [&]() {
+                        if (nb == 0) frag_wait(kf);
+                        acc[q & 1] = chain(nb);
+                        asm volatile("" : "+v"(acc[0]), "+v"(acc[1]));  // the chain stays where it was written
+                        if (nb == NB - 1) {  // this fragment's last chain has been issued: read back the next one
+                            if (na == 0) take_frag(std::integral_constant<int, SLOT * STAGE_BYTES + 32 * ROW_BYTES>{}, kf);
+                            else take_frag(std::integral_constant<int, ((SLOT + 1) % NS) * STAGE_BYTES>{}, kf);
+                        }
+                    };
+                    auto do_drain = [&]() {
+                        if (!have_prev) return;
+                        drain_begin(p_kb, p_na, p_nb);
+                        if (p_fast) drain_fast(acc[(q - 1) & 1]);
+                        else drain_slow(acc[(q - 1) & 1], p_kb, p_na, p_nb);
+                        drain_end(p_nb);
+                        asm volatile("" : "+v"(acc[0]), "+v"(acc[1]));
+                    };
+                    // Chain first: the matrix pipe works on tile q while the VALU exponentiates tile q - 1.
+                    // (Measured slower: the exponent work woven between the chain's MFMAs, and the two waves
+                    // of a SIMD in opposite order.)
+                    do_chain();
+                    do_drain();
+                }
+            };
+            static_assert(NA == 2, "fragment offsets above");
+            for (int st0 = s0; st0 < s1; st0 += NS) {
+                stage(st0, std::integral_constant<int, 0>{});
+                if (st0 + 1 < s1) stage(st0 + 1, std::integral_constant<int, 1>{});
+                if (st0 + 2 < s1) stage(st0 + 2, std::integral_constant<int, 2>{});
+                if (NS > 3 && st0 + 3 < s1) stage(st0 + 3, std::integral_constant<int, 3 % NS>{});
             }
-        };
-        auto drain_end = [&](int nb) {
-            if (nb == NB - 1) {
-                float tot = (cp[0] + cp[1]) + (cp[2] + cp[3]);
-                cp[0] = cp[1] = cp[2] = cp[3] = 0.f;
-                // v_permlane32_swap exchanges the upper half of its first operand with the lower half of
-                // its second: started from two copies of the value, one register then holds the lower
-                // half-wave's values in both halves and the other the upper half-wave's, so their sum is
-                // the total of the two half-waves in every lane.  (Inline assembly: given the same value
-                // twice, the builtin's two results were folded into one.)
-                float x = tot, y = tot;
-                asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
-                tot = x + y;
-                // plain read-modify-write of the wave's own slot (LDS float atomics are slow): the old
-                // value was requested before the exponent work; both half-waves store the same total
-                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(col_old)::"memory");
-                tot += col_old;
-                asm volatile("ds_write_b32 %0, %1" ::"v"(col_ad), "v"(tot) : "memory");
-            }
+            static_assert(NS <= 4, "unrolled above");
+            drain_begin(c0 + (s1 - 1) * KT, NA - 1, NB - 1);
+            drain_slow(acc[(TILES - 1) & 1], c0 + (s1 - 1) * KT, NA - 1, NB - 1);
+            drain_end(NB - 1);
+            // the look-ahead fetches and the operand read-back issued past the last stage must be over before
+            // the ring (and nl_s) is reused by the next phase or unit
+            FCS_WAIT_VM(0);
+            frag_wait(kf);
+            block_sync();
         };
 
-        // MFMA chain of one tile alone
-        auto chain = [&](int nb) {
-            floatx16 c = mfma16<BF>(qf[nb][0], kf[0], cinit[nb]);
-#pragma unroll
-            for (int t = 1; t < NT; ++t) c = mfma16<BF>(qf[nb][t], kf[t], c);
-            return c;
-        };
-        auto drain_fast = [&](const floatx16 &sc) {  // every key of the tile visible, no stabilised row
-#pragma unroll
-            for (int i = 0; i < 16; ++i) cp[i & 3] += fast_exp2(PRE ? sc[i] : sc[i] * cmul);
-        };
-
-        // one stage, in ring slot SLOT (compile-time)
-        auto stage = [&](int st, auto slot_c) {
-            constexpr int SLOT = decltype(slot_c)::value;
-            const int kb = c0 + st * KT;
-            if (st > 0) {
-                // stage st + 1 has landed (this wave's pieces; the barrier extends that to everyone's), and
-                // every wave is done reading stage st - 1, whose slot takes the next fetch
-                FCS_WAIT_VM((NS - 3) * IPW);
-                block_barrier();
-            }
-            fetch_stage(st + NS - 1, (SLOT + NS - 1) % NS);
-#pragma unroll
-            for (int q = 0; q < TILES; ++q) {
-                const int na = q / NB, nb = q % NB;
-                // the previous tile: the one before in this stage, or the last of the previous stage
-                const int p_kb = (q > 0) ? kb : kb - KT;
-                const int p_na = (q > 0) ? (q - 1) / NB : NA - 1, p_nb = (q > 0) ? (q - 1) % NB : NB - 1;
-                const bool have_prev = (q > 0) || (st > 0);
-                const bool p_fast = !shifted && !(p_kb + p_na * 32 + 31 > thr_wave_min);  // wave-uniform
-                auto do_chain = [&]() {
-                    if (nb == 0) frag_wait(kf);
-                    acc[q & 1] = chain(nb);
-                    asm volatile("" : "+v"(acc[0]), "+v"(acc[1]));  // the chain stays where it was written
-                    if (nb == NB - 1) {  // this fragment's last chain has been issued: read back the next one
-                        if (na == 0) take_frag(std::integral_constant<int, SLOT * STAGE_BYTES + 32 * ROW_BYTES>{}, kf);
-                        else take_frag(std::integral_constant<int, ((SLOT + 1) % NS) * STAGE_BYTES>{}, kf);
-                    }
-                };
-                auto do_drain = [&]() {
-                    if (!have_prev) return;
-                    drain_begin(p_kb, p_na, p_nb);
-                    if (p_fast) drain_fast(acc[(q - 1) & 1]);
-                    else drain_slow(acc[(q - 1) & 1], p_kb, p_na, p_nb);
-                    drain_end(p_nb);
-                    asm volatile("" : "+v"(acc[0]), "+v"(acc[1]));
-                };
-                // Chain first: the matrix pipe works on tile q while the VALU exponentiates tile q - 1.
-                // (Measured slower: the exponent work woven between the chain's MFMAs, and the two waves
-                // of a SIMD in opposite order.)
-                do_chain();
-                do_drain();
-            }
-        };
-        static_assert(NA == 2, "fragment offsets above");
-        for (int st0 = 0; st0 < nst; st0 += NS) {
-            stage(st0, std::integral_constant<int, 0>{});
-            if (st0 + 1 < nst) stage(st0 + 1, std::integral_constant<int, 1>{});
-            if (st0 + 2 < nst) stage(st0 + 2, std::integral_constant<int, 2>{});
-            if (NS > 3 && st0 + 3 < nst) stage(st0 + 3, std::integral_constant<int, 3 % NS>{});
+        // (one call site per form of the operand, so that the stream's code exists twice, not three times)
+        int raw0 = 0;  // first stage of the raw phase
+        if (PRE && n_pre > 0) {
+            shape_q(true);
+            run_phase(std::true_type{}, 0, n_pre, true);
+            raw0 = n_pre;
+            if (raw0 < nst) load_q_rows();  // the unit's last stages (causal: keys that not every row sees)
         }
-        static_assert(NS <= 4, "unrolled above");
-        drain_begin(c0 + (nst - 1) * KT, NA - 1, NB - 1);
-        drain_slow(acc[(TILES - 1) & 1], c0 + (nst - 1) * KT, NA - 1, NB - 1);
-        drain_end(NB - 1);
-        // the look-ahead fetches and the operand read-back issued past the last stage must be over before
-        // the next unit reuses the ring (and nl_s)
-        FCS_WAIT_VM(0);
-        frag_wait(kf);
-        block_sync();
+        if (raw0 < nst) {
+            shape_q(false);
+            run_phase(std::false_type{}, raw0, nst, raw0 == 0);
+        }
     }
 
     // ---- add the waves' slices in wave order and store
@@ -493,8 +531,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_colstream_kernel(const Args
 // [2^-80, 2^110); a block that leaves that range redoes its keys in two more sweeps (row maxima, then
 // sums of 2^((s - m) * c), the maximum subtracted before the scale).  Writes (m, log2 l) per row, or
 // (m, l) per (split, row) when the keys are split; the column pass merges the splits.
-// PRE: see the column pass.  The common sweep runs on Q * c rounded to fp16 and accepts row sums below
-// 2^20 only; a block that leaves the range reloads the raw operand for its stabilised sweeps.
+// PRE: see the column pass.  The common sweep runs its stages below a.pre_end on Q * c rounded to fp16 (then the
+// rest on the raw operand) and accepts row sums below 2^20 only; a block that leaves the range reloads the raw
+// operand for its stabilised sweeps.
 template <int D, int NB, int WAVES, bool BF, bool PRE>
 __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args a)
 {
@@ -563,7 +602,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
             }
         }
     };
-    load_q(true);
+    // leading stages of the block that run on the pre-scaled operand in the common sweep (block-uniform)
+    const int n_pre = PRE ? min(nst, max(0, (a.pre_end - kc0) / KT)) : 0;
+    load_q(n_pre > 0);
     const char *kp = reinterpret_cast<const char *>(a.k + (int64_t)b * a.ks_b +
                                                     (int64_t)kv_head(h, a.kv_group, a.kv_magic) * a.ks_h);
     const int64_t k_row_b = a.ks_s * 2;
@@ -610,23 +651,26 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
     float rs[NB][16];      // running per-row value (sum or maximum) over this lane's keys
     float nmax[NB][16];    // -m_i of the rows in accumulator layout (stabilised sum sweep only)
 
-    // One sweep over the block's keys.  MAXOP: rs = max of the visible scores; else rs += 2^(score * c)
-    // over the visible keys.  SHIFT: the row's -m_i (in `nmax`) is added to the score before the scale.  The
-    // accumulators always start at 0, so that every sweep, and the column pass for these rows, sees the
-    // very same score bits.
-    auto sweep = [&](auto max_c, auto shift_c) {
-        constexpr bool MAXOP = decltype(max_c)::value;
-        constexpr bool SHIFT = decltype(shift_c)::value;
-        constexpr bool SCALED = PRE && !MAXOP && !SHIFT;  // the common sweep of the pre-scaled variant
-        constexpr int TILES = NA * NB;
-        static_assert(NA == 2 && TILES % 2 == 0, "fragment offsets and the two alternating accumulators");
+    // One sweep over the stages [s0, s1) of the block's keys.  MAXOP: rs = max of the visible scores; else
+    // rs += 2^(score * c) over the visible keys.  SHIFT: the row's -m_i (in `nmax`) is added to the score before
+    // the scale.  SCALED: the operand in `qf` is the pre-scaled one.  The accumulators always start at 0, so that
+    // every sweep, and the column pass for these rows, sees the very same score bits.
+    auto reset_rows = [&](auto max_c) {
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) rs[nb][i] = MAXOP ? kNegBig : 0.f;
-        if (nst == 0) return;  // block-uniform
+            for (int i = 0; i < 16; ++i) rs[nb][i] = decltype(max_c)::value ? kNegBig : 0.f;
+    };
+    auto sweep = [&](auto max_c, auto shift_c, auto scaled_c, const int s0, const int s1) {
+        constexpr bool MAXOP = decltype(max_c)::value;
+        constexpr bool SHIFT = decltype(shift_c)::value;
+        constexpr bool SCALED = decltype(scaled_c)::value;
+        static_assert(!SCALED || (PRE && !MAXOP && !SHIFT), "only the common sweep of the pre-scaled variant");
+        constexpr int TILES = NA * NB;
+        static_assert(NA == 2 && TILES % 2 == 0, "fragment offsets and the two alternating accumulators");
+        if (s1 <= s0) return;  // block-uniform
 #pragma unroll
-        for (int st = 0; st < NS - 1; ++st) fetch_stage(st, st);
+        for (int st = 0; st < NS - 1; ++st) fetch_stage(s0 + st, st);
         FCS_WAIT_VM((NS - 3) * IPW);
         block_sync();
         take_frag(std::integral_constant<int, 0>{}, kf);
@@ -656,7 +700,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
         auto stage = [&](int st, auto slot_c) {
             constexpr int SLOT = decltype(slot_c)::value;
             const int kb = kc0 + st * KT;
-            if (st > 0) {
+            if (st > s0) {
                 FCS_WAIT_VM((NS - 3) * IPW);
                 block_barrier();
             }
@@ -676,16 +720,16 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
                     else take_frag(std::integral_constant<int, ((SLOT + 1) % NS) * STAGE_BYTES>{}, kf);
                 }
                 if (q > 0) drain(acc[(q - 1) & 1], kb, (q - 1) / NB, (q - 1) % NB);
-                else if (st > 0) drain(acc[(TILES - 1) & 1], kb - KT, NA - 1, NB - 1);
+                else if (st > s0) drain(acc[(TILES - 1) & 1], kb - KT, NA - 1, NB - 1);
             }
         };
-        for (int st0 = 0; st0 < nst; st0 += NS) {
+        for (int st0 = s0; st0 < s1; st0 += NS) {
             stage(st0, std::integral_constant<int, 0>{});
-            if (st0 + 1 < nst) stage(st0 + 1, std::integral_constant<int, 1>{});
-            if (st0 + 2 < nst) stage(st0 + 2, std::integral_constant<int, 2>{});
-            if (NS > 3 && st0 + 3 < nst) stage(st0 + 3, std::integral_constant<int, 3 % NS>{});
+            if (st0 + 1 < s1) stage(st0 + 1, std::integral_constant<int, 1>{});
+            if (st0 + 2 < s1) stage(st0 + 2, std::integral_constant<int, 2>{});
+            if (NS > 3 && st0 + 3 < s1) stage(st0 + 3, std::integral_constant<int, 3 % NS>{});
         }
-        drain(acc[(TILES - 1) & 1], kc0 + (nst - 1) * KT, NA - 1, NB - 1);
+        drain(acc[(TILES - 1) & 1], kc0 + (s1 - 1) * KT, NA - 1, NB - 1);
         FCS_WAIT_VM(0);
         frag_wait(kf);
         block_sync();  // the ring may be refilled by the next sweep
@@ -713,8 +757,13 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
         }
     };
 
-    // ---- common path: no max subtraction
-    sweep(std::false_type{}, std::false_type{});
+    // ---- common path: no max subtraction; the pre-scaled stages first, then the raw ones
+    reset_rows(std::false_type{});
+    if constexpr (PRE) {
+        sweep(std::false_type{}, std::false_type{}, std::true_type{}, 0, n_pre);
+        if (n_pre > 0 && n_pre < nst) load_q(false);
+    }
+    sweep(std::false_type{}, std::false_type{}, std::false_type{}, n_pre, nst);
     float lt[NB], m_row[NB];
     fold_lanes(std::false_type{}, lt);
     bool has[NB], bad = false;
@@ -724,7 +773,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
         const int thr = a.causal ? min(a.k_past + qi, a.Sk - 1) : a.Sk - 1;  // last key this row sees
         has[nb] = (nst > 0) && (kc0 <= thr);
         // ceiling 2^110 rather than 2^120: up to 512 key splits of a row are added up by the column pass
-        bad = bad || (has[nb] && !(lt[nb] >= 8.2718061e-25f && lt[nb] < (PRE ? kRowSumHiPre : 1.2980742e+33f)));
+        bad = bad || (has[nb] && !(lt[nb] >= 8.2718061e-25f && lt[nb] < (n_pre > 0 ? kRowSumHiPre : 1.2980742e+33f)));
         m_row[nb] = has[nb] ? 0.f : kNegBig;  // an empty split must not set the merged maximum
         if (!has[nb]) lt[nb] = 0.f;
     }
@@ -741,7 +790,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
     // ---- rare: row maxima first, then sums with the maximum subtracted before the scale
     if (bad) {
         if (PRE) load_q(false);
-        sweep(std::true_type{}, std::false_type{});
+        reset_rows(std::true_type{});
+        sweep(std::true_type{}, std::false_type{}, std::false_type{}, 0, nst);
         float mx[NB];
         fold_lanes(std::true_type{}, mx);
 #pragma unroll
@@ -754,7 +804,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) nmax[nb][i] = -mrow[wave * ROWS_W + nb * 32 + 8 * (i >> 2) + 4 * g + (i & 3)];
-        sweep(std::false_type{}, std::true_type{});
+        reset_rows(std::false_type{});
+        sweep(std::false_type{}, std::true_type{}, std::false_type{}, 0, nst);
         fold_lanes(std::false_type{}, lt);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
@@ -785,14 +836,18 @@ __global__ __launch_bounds__(64 * WAVES, 2) void fcs_rowstream_kernel(const Args
 // host side
 // ------------------------------------------------------------------------------------
 // Both passes must agree on the pre-scaled variant: fp16 operands, 64-wide kernels, |scale| <= 1/8, and
-// at least 16384 (head, row) pairs averaged into EVERY output (the rounding of Q * c to fp16 perturbs
-// every score by about 2^-12 relative; over that many rows its effect on a mean stays below 2e-4
-// relative at unit-variance inputs).  Causal calls never qualify: their last keys are seen by a handful of rows only, and
-// there the perturbation shows undiminished (measured 1e-3 relative at four times unit-variance inputs).
+// at least 16384 (head, row) pairs averaged into every output that is computed from pre-scaled scores (the
+// rounding of Q * c to fp16 perturbs every score by about 2^-12 relative; over that many rows its effect on a
+// mean stays below 2e-4 relative at unit-variance inputs).  Of a causal call only the keys that every row sees
+// qualify, in whole 64-key stages (Args::pre_end): its last keys are seen by a handful of rows only, and there the
+// perturbation shows undiminished (measured 1e-3 relative at four times unit-variance inputs).
+// (128-wide heads gain nothing from it: there the matrix pipe has twice the work per score and the kernels are no
+// longer bound by the exponent's VALU work alone: B 1, H 16, S 8192, D 128 548 against 552 us, the causal
+// H 32, Q 512, K 65536, D 128 622 against 610 us.)
 static bool stream_prescaled(const Plan &p, const Args &a)
 {
-    return !p.bf16 && !p.causal && p.Dp == 64 && a.c != 0.f && fabsf(a.c) <= 0.1251f * 1.44269504f &&
-           (long)p.H * p.q_rows >= 16384;
+    return !p.bf16 && p.Dp == 64 && a.c != 0.f && fabsf(a.c) <= 0.1251f * 1.44269504f && (long)p.H * p.q_rows >= 16384 &&
+           a.pre_end >= 4 * kStageKeys;
 }
 
 template <int D, int NB, int WAVES, bool BF>

@@ -278,7 +278,14 @@ def test_prescaled_shared_q_variant(shape, same, kw, boost):
     ((1, 4, 4096, 64), (1, 4, 4096, 64), {}, False, 0.0),                        # non-causal, keys split in pass 1
     ((1, 4, 4096, 64), (1, 4, 4096, 64), {"scale": -0.125}, False, 0.0),         # the sign rides on the operand
     ((2, 8, 2100, 64), (2, 8, 2100, 64), {}, False, 0.0),                        # ragged, just past the fused kernel's range
-    ((1, 16, 700, 64), (1, 16, 5000, 64), {"is_causal": True}, False, 0.0),      # causal: always the exact variant
+    ((1, 16, 700, 64), (1, 16, 5000, 64), {"is_causal": True}, False, 0.0),      # causal, 11200 pairs: the exact variant
+    ((1, 16, 1100, 64), (1, 16, 5000, 64), {"is_causal": True}, False, 0.0),     # causal, 17600 pairs: pre-scaled below key 3840
+    ((1, 16, 1100, 64), (1, 16, 5000, 64), {"is_causal": True}, False, 6.0),     # ... with rows that leave the 2^20 range
+    ((1, 32, 512, 64), (1, 32, 9000, 64), {"is_causal": True}, False, 0.0),      # causal, two phases per unit
+    ((1, 32, 512, 64), (1, 32, 9000, 64), {"is_causal": True, "scale": -0.08}, False, 0.0),
+    ((1, 32, 512, 40), (1, 32, 8704, 40), {"is_causal": True}, False, 6.0),      # k_past a multiple of 64; narrower head
+    ((1, 4, 8192, 64), (1, 4, 64, 64), {"is_causal": True}, False, 0.0),         # more rows than keys: no key is seen by every row
+    ((1, 8, 2200, 128), (1, 8, 2200, 128), {}, False, 0.0),                      # 128-wide heads: the exact variant
     ((2, 8, 2500, 48), (2, 8, 2500, 48), {}, False, 0.0),                        # narrower head in the 64-wide kernels
     ((1, 8, 3000, 64), (1, 8, 3000, 64), {"cls_len": 2500}, False, 0.0),         # 20000 averaged pairs
     ((1, 4, 3000, 64), (1, 4, 3000, 64), {"cls_len": 1500}, False, 0.0),         # 6000 averaged pairs: the exact variant
@@ -289,15 +296,23 @@ def test_prescaled_shared_q_variant(shape, same, kw, boost):
     ((1, 2, 4096, 64), (1, 2, 4096, 64), {}, False, 0.0),                        # fewer than 16384 pairs: the exact variant
 ])
 def test_prescaled_streaming_variant(qs, ks, kw, same, boost):
-    """Non-causal two-pass calls with fp16 operands, 64-wide kernels, |scale| <= 1/8 and >= 16384 averaged
-    (head, row) pairs run both passes on Q * c rounded to fp16; blocks whose row sums reach 2^20 (or fall below
-    2^-80) must redo their keys on the raw operand, and the column pass must follow them there."""
+    """Two-pass calls with fp16 operands, 64-wide kernels, |scale| <= 1/8 and >= 16384 averaged
+    (head, row) pairs run both passes on Q * c rounded to fp16 for the keys that every row sees (all keys of a
+    non-causal call; whole 64-key stages below k_past of a causal one, whose last keys keep the raw operand);
+    blocks whose row sums reach 2^20 (or fall below 2^-80) must redo their keys on the raw operand, and the column
+    pass must follow them there.  The last Q_len columns of a causal call, averaged over few rows each, are
+    checked on their own."""
     q, k = _inputs(qs, ks, seed=13, same=same)
     if boost:
         q[:, 1, 100:164] *= boost
         if same:
             k = q.clone()
-    _assert_close(_run(q, k, **kw), _oracle(q, k, **kw), f"prescaled streaming {qs} {ks} {kw} same={same} boost={boost}")
+    out, ref = _run(q, k, **kw), _oracle(q, k, **kw)
+    what = f"prescaled streaming {qs} {ks} {kw} same={same} boost={boost}"
+    _assert_close(out, ref, what)
+    if kw.get("is_causal") and ks[2] > qs[2]:
+        _assert_close(out[:, -qs[2]:], ref[:, -qs[2]:], what + " (diagonal window)")
+        _assert_close(out[:, : ks[2] - qs[2]], ref[:, : ks[2] - qs[2]], what + " (keys every row sees)")
 
 
 @pytest.mark.parametrize("amp", [1.0, 1.6, 2.0, 2.5])
@@ -310,6 +325,11 @@ def test_prescaled_variants_against_input_amplitude(amp):
         q = (torch.randn(shape, generator=g) * amp).half()
         k = (torch.randn(shape, generator=g) * amp).half()
         _assert_close(_run(q, k, scale=0.125), _oracle(q, k, scale=0.125), f"amplitude {amp} {shape}")
+    # the streaming kernels' pre-scaled variant on a causal call (the keys below k_past)
+    g = torch.Generator().manual_seed(6)
+    q = (torch.randn((1, 16, 1024, 64), generator=g) * amp).half()
+    k = (torch.randn((1, 16, 6000, 64), generator=g) * amp).half()
+    _assert_close(_run(q, k, scale=0.125, is_causal=True), _oracle(q, k, scale=0.125, is_causal=True), f"amplitude {amp} causal")
 
 
 @pytest.mark.parametrize("qs,ks,kw", [

@@ -200,6 +200,11 @@ def test_plan_description_and_k_past_clamp():
     assert "fcs_fewrows_kernel<64,1,false>" in d((32, 16, 577, 64), (32, 16, 577, 64), cls_n=1)
     t = d((1, 32, 512, 128), (1, 32, 65536, 128), causal=True)
     assert "fcs_rowstream_kernel<128,2,8,false,false>" in t and "fcs_colstream_kernel<128,2,8,false,false>" in t
+    # 64-wide heads, 32 x 512 = 16384 averaged rows: both passes on the pre-scaled operand for the keys every row sees
+    t = d((1, 32, 512, 64), (1, 32, 65536, 64), causal=True)
+    assert "fcs_rowstream_kernel<64,2,8,false,true>" in t and "fcs_colstream_kernel<64,2,8,false,true>" in t
+    t = d((1, 32, 128, 64), (1, 32, 4096, 64), causal=True)
+    assert "fcs_rowstream_kernel<64,1,4,false,false>" in t and "fcs_colstream_kernel<64,1,4,false,false>" in t
     assert "bf16" not in t and "fcs_fused_kernel<64,8,true,8,true,false>" in d((8, 16, 2048, 64), (8, 16, 2048, 64), bf16=True)
     base = d((1, 4, 100, 128), (1, 4, 1000, 128), causal=True, k_past=1000)
     for kp in (1001, 5000, 2 ** 31 - 1, 2 ** 40):
