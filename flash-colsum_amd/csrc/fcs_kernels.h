@@ -39,7 +39,7 @@ struct Args {
     // fused single-kernel path (scores stay in registers)
     int f_kg;        // waves along the key axis (1, 2, 4 or 8); 8 / f_kg waves along the query axis
     int f_tpw;       // 32-key tiles per wave (<= 8)
-    int f_nqblk;     // blocks along the query axis (32 * 8 / f_kg rows each)
+    int f_nqblk;     // blocks along the query axis (32 * 8 / f_kg rows each; short-sequence path: 32-row tiles per head)
     int f_hpg;       // heads per block
     int f_rbpw;      // adjacent row blocks per block (a block walks over f_rbpw x f_hpg units)
     int f_nwgq;      // blocks along the query axis: ceil(f_nqblk / f_rbpw)
@@ -53,6 +53,8 @@ int launch_colsum(const Plan &p, const Args &a, void *stream);
 hipError_t launch_fused(const Plan &p, const Args &a, hipStream_t st);
 // few-rows path (fcs_fewrows.hip): p.fewrows == 1
 hipError_t launch_fewrows(const Plan &p, const Args &a, hipStream_t st);
+// short-sequence path (fcs_small.hip): p.small == 1
+hipError_t launch_small(const Plan &p, const Args &a, hipStream_t st);
 
 // row-statistics pass and column pass of the two-pass path (fcs_stream.hip)
 hipError_t launch_rowstream(const Plan &p, const Args &a, hipStream_t st);
@@ -65,6 +67,7 @@ hipError_t launch_finalize(const Args &a, hipStream_t st);
 size_t describe_colsum(const Plan &p, const Args &a, char *buf, size_t n);
 size_t describe_fused(const Plan &p, const Args &a, char *buf, size_t n);
 size_t describe_fewrows(const Plan &p, const Args &a, char *buf, size_t n);
+size_t describe_small(const Plan &p, const Args &a, char *buf, size_t n);
 size_t describe_two_pass(const Plan &p, const Args &a, char *buf, size_t n);
 size_t describe_finalize(const Args &a, char *buf, size_t n);
 

@@ -98,6 +98,7 @@ int launch_colsum(const Plan &p, const Args &a, void *stream)
 {
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (p.fewrows) return (int)launch_fewrows(p, a, st);
+    if (p.small) return (int)launch_small(p, a, st);
     if (p.fused) return (int)launch_fused(p, a, st);
     return (int)launch_two_pass(p, a, st);
 }
@@ -105,6 +106,7 @@ int launch_colsum(const Plan &p, const Args &a, void *stream)
 size_t describe_colsum(const Plan &p, const Args &a, char *buf, size_t n)
 {
     if (p.fewrows) return describe_fewrows(p, a, buf, n);
+    if (p.small) return describe_small(p, a, buf, n);
     if (p.fused) return describe_fused(p, a, buf, n);
     return describe_two_pass(p, a, buf, n);
 }

@@ -13,6 +13,9 @@ constexpr int kComputeUnits = 256;  // MI355X
 constexpr int kFusedMaxKeys = 2048; // 8 waves x 8 tiles x 32 keys of fp32 scores per 32 query rows
 constexpr int kFewRowsMaxRows = 4;      // few-rows path: at most this many averaged query rows per head ...
 constexpr int kFewRowsMaxScores = 12288; // ... and rows * Sk scores (48 KB of LDS)
+constexpr int kSmallMaxTiles = 9;        // short-sequence path: one wave holds the scores of 32 rows x (32 x 9) keys
+// ... whose workgroups keep the keys of this many heads in an LDS ring (112 KB at most)
+constexpr int small_ring_heads(int tiles) { return 28 / tiles < 16 ? 28 / tiles : 16; }
 
 // column pass (fcs_stream.hip): ring slots of 64-key stages and keys per workgroup chunk, sized so
 // that the LDS ring plus one accumulator slice per wave fit (twice per compute unit for 4-wave blocks)
@@ -44,6 +47,8 @@ struct Plan {
     // fused single-kernel path: non-causal, all keys of a row block fit in one
     // workgroup's registers.  grid = (f_nwgq * B, f_hg)
     int fewrows;     // 1: few-rows path (non-causal, q_rows <= 4): grid = B * f_hg, slabs = f_hg
+    int small;       // 1: short-sequence path (non-causal, Sk <= 288, D <= 64): grid = B * f_hg, slabs = f_hg,
+                     //    f_tpw key tiles, f_nqblk row tiles of 32 rows per head
     int fused;       // 1: use it (then the two-pass fields above are unused)
     int f_kg, f_qg;  // waves along keys / along queries, f_kg * f_qg == 8
     int f_tpw;       // 32-key tiles per wave
@@ -160,6 +165,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
 
     // ---- few-rows path: a batch of matrix-vector products, one workgroup per (batch entry, head group)
     p.fewrows = 0;
+    p.small = 0;
     p.fused = 0;
     // (One workgroup streams a whole key head and computes its R x Sk scores on the VALU.  The fused
     // path, which splits a head's keys over eight waves and uses the matrix pipe, is quicker when
@@ -183,6 +189,44 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
         p.off_lse = p.off_ml = p.off_partial = 0;
         p.total = align256(sizeof(float) * (size_t)p.n_partials * B * Sk);
         return (long)B * p.f_hg < (1L << 31);
+    }
+
+    // ---- short-sequence path: a wave holds all the keys of its 32 rows, a workgroup owns f_hpg heads of a
+    // batch entry and deals their (head, 32-row tile) items to its eight waves, eight per step
+    if (!causal && Sk <= 32 * kSmallMaxTiles && D <= 64) {
+        const int tiles = ceil_div(Sk, 32), rt = ceil_div(p.q_rows, 32);
+        // the keys of the heads that two consecutive steps touch must fit the ring: items 8t .. 8t + 15
+        int span = 0;
+        for (int t = 0; t < rt; ++t) {
+            const int c = (8 * t + 15) / rt - (8 * t) / rt + 1;
+            if (c > span) span = c;
+        }
+        if (span <= small_ring_heads(tiles)) {
+            p.small = 1;
+            p.f_tpw = tiles;
+            p.f_nqblk = rt;
+            // Heads per workgroup: one workgroup is resident per compute unit, so the launch runs in generations
+            // of kComputeUnits workgroups, each as long as its steps plus about one step for starting and finishing.
+            p.f_hpg = H;
+            double best = 0.;
+            for (int hg = 1, hpg = H; hpg >= 1; hg = (hpg > 1) ? ceil_div(H, hpg - 1) : H + 1, hpg = (hg <= H) ? ceil_div(H, hg) : 0) {
+                const long gens = ((long)B * hg + kComputeUnits - 1) / kComputeUnits;
+                const double cost = (double)gens * (ceil_div(hpg * rt, 8) + 1.0) + 0.01 * hg;
+                if (hg == 1 || cost < best) {
+                    best = cost;
+                    p.f_hpg = hpg;
+                }
+            }
+            p.f_hg = ceil_div(H, p.f_hpg);
+            p.f_rbpw = 1;
+            p.f_nwgq = 1;
+            p.f_kg = 1;
+            p.f_qg = 8;
+            p.n_partials = p.f_hg;
+            p.off_lse = p.off_ml = p.off_partial = 0;
+            p.total = align256(sizeof(float) * (size_t)p.n_partials * B * Sk);
+            return (long)B * p.f_hg < (1L << 31);
+        }
     }
 
     // ---- fused path

@@ -944,6 +944,64 @@ def test_key_tiles_kept_between_row_blocks(qs, ks, kw):
     assert torch.equal(out, _run_ext(q, k, **kw)), "not reproducible"
 
 
+@pytest.mark.parametrize("shape,d,kw,bf16,boost", [
+    ((64, 12, 197, 64), 64, {}, False, 0.0),                    # ViT-B/16: 7 row tiles x 7 key tiles, pre-scaled
+    ((32, 16, 257, 64), 64, {}, False, 0.0),                    # CLIP ViT-L/14: nine key tiles, one key in the last
+    ((8, 16, 256, 64), 64, {}, False, 0.0),                     # whole tiles, 4096 averaged rows exactly
+    ((8, 16, 256, 64), 64, {"scale": -0.125}, False, 0.0),
+    ((4, 5, 288, 64), 64, {}, False, 0.0),                      # the longest this path takes; five heads in groups
+    ((3, 7, 100, 64), 64, {}, False, 0.0),                      # fewer than 4096 averaged rows: exact operand
+    ((3, 7, 100, 64), 64, {"scale": 0.3}, True, 0.0),
+    ((2, 3, 1, 64), 64, {}, False, 0.0),                        # a single key (one row: the few-rows kernel)
+    ((2, 9, 5, 64), 64, {}, False, 0.0),                        # five keys in one tile
+    ((2, 40, 31, 64), 64, {}, False, 0.0),
+    ((2, 40, 33, 64), 64, {}, True, 0.0),
+    ((16, 12, 197, 32), 32, {}, False, 0.0),                    # narrower heads: zero channels
+    ((16, 12, 197, 48), 48, {}, True, 0.0),
+    ((5, 8, 224, 8), 8, {"scale": 0.5}, False, 0.0),
+    ((6, 24, 197, 64), 64, {"cls_len": 100}, False, 0.0),       # four row tiles of a head, seven key tiles
+    ((6, 24, 197, 64), 64, {"cls_len": 33}, False, 0.0),        # two row tiles: the ring would not hold the heads of a step -> longer kernel
+    ((16, 16, 256, 64), 64, {}, False, 6.0),                    # rows that leave the pre-scaled range: exact path inside the kernel
+    ((16, 16, 197, 64), 64, {}, False, 40.0),                   # ... and the unstabilised range altogether
+    ((2, 4, 257, 64), 64, {}, True, 40.0),
+])
+def test_short_sequences_single_wave_kernel(shape, d, kw, bf16, boost):
+    """Non-causal calls with at most 288 keys and head dims up to 64: one wave holds the scores of 32 rows and all
+    keys, the keys of a head are fetched once per workgroup.  Dense and (B,S,H,D) storage give the same bits."""
+    from flash_colsum import _hip
+
+    g = torch.Generator().manual_seed(51)
+    q = torch.randn(shape, generator=g)
+    k = torch.randn(shape, generator=g)
+    if boost:
+        q[:, 1, 10:40] *= boost
+    q, k = (q.bfloat16(), k.bfloat16()) if bf16 else (q.half(), k.half())
+    print("short sequence", shape, kw, _hip.plan_description(shape, shape, cls_n=kw.get("cls_len", -1), scale=kw.get("scale"), bf16=bf16),
+          flush=True)
+    ref = _oracle(q.float(), k.float(), **kw)
+    out = _run(q, k, **kw)
+    _assert_close(out, ref, f"short {shape} {kw} bf16={bf16} boost={boost}")
+    assert torch.equal(out, _run(q, k, **kw))
+    qs = q.cuda().permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)  # (B,S,H,D) storage
+    ks = k.cuda().permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    assert torch.equal(out, _run(qs, ks, **kw))
+
+
+def test_short_sequences_with_grouped_heads_and_unequal_lengths():
+    """The same kernel behind flash_colsum_ext: grouped key heads, S_q != S_k."""
+    from flash_colsum import flash_colsum_ext
+    from oracle import colsum_ext_exact
+
+    g = torch.Generator().manual_seed(52)
+    for qs, ks, kw in [((3, 8, 197, 64), (3, 2, 197, 64), {}), ((2, 6, 500, 64), (2, 6, 100, 64), {}),
+                       ((2, 12, 40, 32), (2, 3, 288, 32), {"cls_len": 37}), ((1, 4, 1000, 64), (1, 1, 257, 64), {"scale": -0.1})]:
+        q = torch.randn(qs, generator=g).half()
+        k = torch.randn(ks, generator=g).half()
+        out = flash_colsum_ext(q.cuda(), k.cuda(), out_dtype=torch.float32, **kw)
+        torch.cuda.synchronize()
+        _assert_close(out, colsum_ext_exact(q, k, **kw), f"short ext {qs} {ks} {kw}")
+
+
 @pytest.mark.parametrize("s_k", [31, 32, 33, 47, 63, 64, 65, 95, 97, 255, 257, 1055, 1100, 1793, 2047])
 def test_last_key_tile_ends_at_the_last_key(s_k):
     """The fused kernel fetches 32-key tiles; a tile that would reach past the last key is moved back

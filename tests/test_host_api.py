@@ -153,9 +153,9 @@ def test_argument_errors_are_reported_without_a_gpu():
 def _call_struct(**kw):
     c = _hip._Call()
     c.struct_bytes = ctypes.sizeof(_hip._Call)
-    c.dtype, c.causal, c.B, c.Hq, c.Hk, c.Sq, c.Sk, c.D, c.cls_n, c.k_past, c.scale = 0, 0, 2, 8, 8, 16, 16, 64, -1, 0, 0.125
-    c.q_strides = (ctypes.c_int64 * 4)(8 * 16 * 64, 16 * 64, 64, 1)
-    c.k_strides = (ctypes.c_int64 * 4)(8 * 16 * 64, 16 * 64, 64, 1)
+    c.dtype, c.causal, c.B, c.Hq, c.Hk, c.Sq, c.Sk, c.D, c.cls_n, c.k_past, c.scale = 0, 0, 2, 8, 8, 1024, 1024, 64, -1, 0, 0.125
+    c.q_strides = (ctypes.c_int64 * 4)(8 * 1024 * 64, 1024 * 64, 64, 1)
+    c.k_strides = (ctypes.c_int64 * 4)(8 * 1024 * 64, 1024 * 64, 64, 1)
     c.q = c.k = c.out = c.ws = 4096  # never dereferenced
     c.ws_bytes = 1 << 30
     for name, v in kw.items():
@@ -198,6 +198,13 @@ def test_plan_description_and_k_past_clamp():
     t = d((8, 16, 2048, 64), (8, 16, 2048, 64))
     assert "fcs_fused_kernel<64,8,false,8,false,true>" in t and "fcs_finalize_kernel<8>" in t
     assert "fcs_fewrows_kernel<64,1,false>" in d((32, 16, 577, 64), (32, 16, 577, 64), cls_n=1)
+    # short sequences: one wave per 32 rows; three heads per workgroup fill the 256 compute units at B 64, H 12
+    t = d((64, 12, 197, 64), (64, 12, 197, 64))
+    assert "fcs_small_kernel<7,false,true> grid 256, 3 heads x 7 row tiles" in t, t
+    assert "fcs_small_kernel<9,true,false>" in d((32, 16, 257, 64), (32, 16, 257, 64), bf16=True)
+    assert "fcs_small_kernel<1,false,false>" in d((2, 3, 5, 40), (2, 3, 5, 40))
+    assert "fcs_fused_kernel" in d((6, 24, 197, 64), (6, 24, 197, 64), cls_n=33)  # two row tiles per head: too many heads per step
+    assert "fcs_fused_kernel" in d((2, 4, 289, 64), (2, 4, 289, 64))
     t = d((1, 32, 512, 128), (1, 32, 65536, 128), causal=True)
     assert "fcs_rowstream_kernel<128,2,8,false,false>" in t and "fcs_colstream_kernel<128,2,8,false,false>" in t
     # 64-wide heads, 32 x 512 = 16384 averaged rows: both passes on the pre-scaled operand for the keys every row sees
@@ -209,10 +216,10 @@ def test_plan_description_and_k_past_clamp():
     base = d((1, 4, 100, 128), (1, 4, 1000, 128), causal=True, k_past=1000)
     for kp in (1001, 5000, 2 ** 31 - 1, 2 ** 40):
         assert d((1, 4, 100, 128), (1, 4, 1000, 128), causal=True, k_past=kp) == base
-    c = _call_struct(causal=1, Sq=100, Sk=1000, k_past=2 ** 31 - 1)
+    c = _call_struct(causal=1, Sq=100, k_past=2 ** 31 - 1)
     buf = ctypes.create_string_buffer(1024)
     n = _hip.lib().fcs_plan_describe(ctypes.byref(c), buf, len(buf))
-    c.k_past = 1000
+    c.k_past = 1024
     buf2 = ctypes.create_string_buffer(1024)
     assert n > 0 and _hip.lib().fcs_plan_describe(ctypes.byref(c), buf2, len(buf2)) == n and buf.value == buf2.value
     # snprintf semantics: truncated output, full length returned
