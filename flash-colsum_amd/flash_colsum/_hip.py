@@ -251,6 +251,42 @@ def _enqueue(causal, q, k, scale, cls_n, k_past, want_f16, f16_only=False):
     return (out, out_h) if want_f16 else out
 
 
+_FP16_MAX = 65504.0
+
+
+def _wide_operands(q: torch.Tensor, k: torch.Tensor):
+    """fp32 / fp64 operands.  The kernels' operand types are fp16 and bf16; the reference's kernels upcast whatever
+    they are given (reference: flash_colsum/kernel_noncausal_batched.py:30-37,47-54, kernel_causal.py:26-32).
+    Values inside fp16's range are rounded to fp16 (the mantissa of the reference's TF32 products).  Larger ones
+    would become inf there: they run on the bf16 kernels instead, each operand split into a high and a low bf16
+    part (16 mantissa bits together) laid side by side along the head dim, Q as [hi, hi, lo, lo] and K as
+    [hi, lo, hi, lo], so that one dot product over 4 D channels adds up all four partial products.  That needs
+    4 D <= 256; wider heads raise.  The range test reads one number back from the GPU; while a stream is
+    capturing a graph it is skipped and the operands are rounded to fp16 unseen."""
+    if torch.cuda.is_current_stream_capturing():
+        return q.to(torch.float16), k.to(torch.float16), torch.float16
+    amax = max(float(t.detach().abs().max()) if t.dtype not in (torch.float16, torch.bfloat16) else 0.0 for t in (q, k))
+    if amax <= _FP16_MAX:  # (a NaN or an infinity fails this test too)
+        return q.to(torch.float16), k.to(torch.float16), torch.float16
+    if amax != amax or amax == float("inf"):
+        raise ValueError("query / key hold NaN or infinite values")
+    d = q.shape[-1]
+    if 4 * d > _MAX_HEAD_DIM or d != k.shape[-1]:
+        raise ValueError(
+            f"query / key values reach {amax:.6g}, beyond fp16's range (+-{_FP16_MAX:g}); with head_dim {d} > "
+            f"{_MAX_HEAD_DIM // 4} they cannot be split into bf16 parts either: pass bfloat16 tensors (same range "
+            "as fp32, 8 mantissa bits) or rescale the operands and `scale`")
+
+    def split(t):
+        t = t.float()
+        hi = t.bfloat16()
+        return hi, (t - hi.float()).bfloat16()
+
+    q_hi, q_lo = split(q)
+    k_hi, k_lo = split(k)
+    return torch.cat([q_hi, q_hi, q_lo, q_lo], dim=-1), torch.cat([k_hi, k_lo, k_hi, k_lo], dim=-1), torch.bfloat16
+
+
 def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n: int, k_past: int, want_f16: bool = False,
             f16_only: bool = False):
     """Enqueue one call; returns the fp32 means, (fp32, fp16) when `want_f16`, or the fp16 tensor alone
@@ -258,8 +294,12 @@ def _launch(causal: bool, q: torch.Tensor, k: torch.Tensor, scale: float, cls_n:
     want_f16 = want_f16 or f16_only
     if q.device.type != "cuda" or k.device != q.device:
         raise ValueError(f"query and key must live on the same GPU, got {q.device} and {k.device}")
-    # bf16 inputs run natively when both are bf16; every other dtype is converted to fp16
-    dtype = torch.bfloat16 if (q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16) else torch.float16
+    # fp16 and bf16 run natively (a mix of the two as fp16); wider types are rounded or split
+    half = (torch.float16, torch.bfloat16)
+    if q.dtype in half and k.dtype in half:
+        dtype = torch.bfloat16 if (q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16) else torch.float16
+    else:
+        q, k, dtype = _wide_operands(q, k)
     # The library takes head dims that are a multiple of 8 (16-byte rows) up to 256 as they are.  Only a
     # head dim that is not a multiple of 8 is padded with zero channels to the next one (a copy), which
     # leaves every score unchanged; the caller's scale already reflects the real D.

@@ -15,7 +15,8 @@ import torch
 pytestmark = pytest.mark.gpu
 
 ATOL, RTOL = 1e-4, 1e-3
-FACTOR = 16.0  # large-score cases: allowed multiple of the fp32 eager reference's own distance from float64
+FACTOR = 12.0  # large-score cases: allowed multiple of the fp32 eager reference's own distance from float64
+               # (measured: 4 .. 8 with 64-wide kernels, up to 11.6 with 128-wide ones, whose scores take eight chained MFMA steps)
 
 
 def _inputs(qs, ks, seed=0, same=False):
@@ -373,6 +374,31 @@ def test_other_input_dtypes_are_converted_to_fp16():
     _assert_close(flash_colsum_f32(q.cuda().double(), k.cuda().half()), ref, "fp64 / fp16 inputs")
     _assert_close(flash_colsum_f32(q.half().bfloat16().cuda(), k.half().cuda()),
                   _oracle(q.half().bfloat16().half(), k.half()), "bf16 / fp16 inputs")
+
+
+def test_fp32_operands_beyond_the_fp16_range():
+    """fp32 operands that fp16 cannot hold run on the bf16 kernels as a high + low split (head dims up to 64);
+    wider heads raise a ValueError that names the range."""
+    from flash_colsum import flash_colsum_f32
+
+    g = torch.Generator().manual_seed(61)
+    for shape, kw in [((2, 4, 300, 64), {}), ((1, 3, 100, 32), {"cls_len": 40}), ((1, 2, 64, 64), {"is_causal": True})]:
+        q = torch.randn(shape, generator=g) * 300.0   # |q| up to ~1500, fine for fp16 ...
+        k = torch.randn(shape, generator=g) * 300.0
+        k[..., 3] *= 300.0                            # ... but this channel of K reaches ~4e5
+        scale = 4e-8
+        assert k.abs().max().item() > 65504
+        ref = _oracle(q.double(), k.double(), scale=scale, **kw)
+        out = flash_colsum_f32(q.cuda(), k.cuda(), scale=scale, **kw)
+        torch.cuda.synchronize()
+        _assert_close(out, ref, f"fp32 beyond fp16 {shape} {kw}")
+    q = torch.randn((1, 2, 50, 128), generator=g)
+    k = torch.randn((1, 2, 50, 128), generator=g) * 1e6
+    with pytest.raises(ValueError, match="beyond fp16's range"):
+        flash_colsum_f32(q.cuda(), k.cuda())
+    k[0, 0, 0, 0] = float("inf")
+    with pytest.raises(ValueError, match="NaN or infinite"):
+        flash_colsum_f32(q.cuda(), k.cuda())
 
 
 @pytest.mark.parametrize("d", [8, 32, 40, 80, 96, 160, 192, 256, 20, 100])
