@@ -44,6 +44,10 @@ constexpr float kSumLo = 8.2718061e-25f;  // 2^-80
 constexpr float kSumHi = 1.3292280e+36f;  // 2^120
 constexpr float kSumHiPre = 268435456.f;  // 2^28: ceiling of the pre-scaled variant (bounds its score rounding error)
 
+// source of the 16-byte pieces that lie past the tensor's head dim (kernels compiled for a wider head); 4 KB, so
+// that a DMA instruction's immediate offset (up to 3 KB) stays inside
+__device__ __attribute__((aligned(16))) unsigned int g_fused_zeros[1024];
+
 #define FCS_GLDS16(gptr, lptr)                                                                \
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gptr), \
                                      (__attribute__((address_space(3))) void *)(lptr), 16, 0, 0)
@@ -149,13 +153,20 @@ __device__ __forceinline__ floatx4 row_values(const RowRed &rr, int i4, int g)
 //                 each score by ~2^-12 relative; the launcher only picks this variant when at least
 //                 4096 (head, row) pairs are averaged per output, where the effect on the means is
 //                 below 1e-4 relative (measured 6.5e-5 at B8 H16 S2048).
-template <int D, int TPW, bool RAGGED, int PRE, bool BF, bool QS = true>
+// NARROW (only on the ragged private-ring variant): the tensor's head dim is smaller than the kernel's D (any
+//                 multiple of 8): the operand pieces past it are fetched from a zero constant.
+template <int D, int TPW, bool RAGGED, int PRE, bool BF, bool QS = true, bool NARROW = false>
 __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
 {
-    static_assert(D == 64, "the fused path is laid out for 64-wide heads");
+    static_assert(!NARROW || (RAGGED && PRE == 0), "narrower heads run on the ragged private-ring variant");
+    static_assert(D == 64 || (D == 128 && PRE == 0 && RAGGED), "64-wide heads, or 128-wide ones on the private-ring ragged variant");
     static_assert(!(PRE && QS && BF), "the pre-scaled variant rounds Q*c to fp16; bf16 would be too coarse");
     constexpr bool PRESCALED = PRE && QS;  // scores leave the MFMAs in the exponent's unit
-    constexpr int NT = D / 16;             // MFMA steps (and 16-byte pieces per lane) per operand tile
+    // A 128-wide head is handled as DC = 2 chunks of 64 channels: an operand tile travels as two half tiles
+    // (32 rows x 64 channels, 4 KB, its own ring item each), and the MFMA chain of a score tile runs over the
+    // first chunk's four steps, then the second chunk's, into the same accumulators.
+    constexpr int DC = D / 64;
+    constexpr int NT = 4;                  // MFMA steps (and 16-byte pieces per lane) per (half) tile
     // KEEP (shared-Q variants with five to eight key tiles per wave): the Q item of those variants is
     // a plain load that needs no ring slot, so the ring holds key tiles only, tile k of every unit in
     // slot k % NS.  The row blocks of a head, which a workgroup walks one after the other, use the
@@ -172,10 +183,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     constexpr bool KEEP_ROT = PRE && (TPW == 6 || (TPW == 8 && PRE != 2));
     constexpr bool KEEP_REV = PRE && !KEEP_ROT;
     constexpr bool KEEP = KEEP_ROT || KEEP_REV;
-    constexpr int NS = KEEP_ROT ? TPW / 2 : KEEP_REV ? (PRE == 2 ? 3 : 4) : 3;  // ring slots per wave
+    // (two chunks: a unit starts by taking three items at once, both Q chunks and the first key half tile, so the
+    // ring holds four, which leaves the fourth in flight)
+    constexpr int NS = KEEP_ROT ? TPW / 2 : KEEP_REV ? (PRE == 2 ? 3 : 4) : (DC == 2 ? 4 : 3);  // ring slots per wave
     constexpr int QV = (PRE == 2) ? 2 : 1;  // load instructions of a wave's share of the raw Q rows
     static_assert(!PRE || (TPW >= 5 && TPW <= 8), "the shared-Q variants are written for five to eight key tiles per wave");
-    constexpr int ITEMS = TPW + 1;         // per (head, row block): the Q tile, then TPW key tiles
+    constexpr int ITEMS = DC * (TPW + 1);  // per (head, row block): the Q tile, then TPW key tiles (chunk by chunk)
     constexpr int SLOT_BYTES = NT * 1024;  // one item: NT pieces x 64 lanes x 16 bytes
     constexpr bool STATIC_SLOTS = KEEP_ROT || (!KEEP_REV && ITEMS % NS == 0);  // then an item's slot is a compile-time value
     __shared__ __attribute__((aligned(16))) char ring[8 * NS * SLOT_BYTES];
@@ -237,8 +250,9 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // so instruction tt reads exactly 1 KB behind instruction tt - 2 and the offsets of instructions
     // 0 and 1 serve all four.  Ragged kernel (key tiles): rows have any pitch, so each instruction has
     // its own offset; it is stored less tt KB, because the instruction's immediate offset (which the
-    // hardware adds to the LDS address AND the global address) supplies tt KB again.  (Never negative:
-    // a row is at least 128 bytes.)
+    // hardware adds to the LDS address AND the global address) supplies tt KB again.  (Never negative
+    // where it is used: heads of 64 channels or more, whose rows are at least 128 bytes; narrower heads form
+    // their offsets at the fetch.)
     auto ragged_voff = [&](int l, uint32_t row_b, int tt) {
         return (uint32_t)(dma_row(l) + 8 * tt) * row_b + dma_piece_b(l, tt & 1) - (uint32_t)(tt * 1024);
     };
@@ -247,6 +261,17 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     uint32_t k_voff[NVOFF];
 #pragma unroll
     for (int i = 0; i < NVOFF; ++i) k_voff[i] = RAGGED ? ragged_voff(lane, k_row_b, i) : dma_row(lane) * k_row_b + dma_piece_b(lane, i);
+    // NARROW: the lane offsets of a key tile's last chunk, instruction by instruction (no immediate-offset trick:
+    // rows may be shorter than 128 bytes).  A piece past the head dim is replaced by the chunk's first piece of the
+    // same row: the Q operand holds zeros in those channels (fetch_ragged_q), so whatever finite values stand in
+    // for the key's add nothing to a score.
+    uint32_t k_voff_n[NARROW ? NT : 1];
+#pragma unroll
+    for (int i = 0; i < (NARROW ? NT : 1); ++i) {
+        const uint32_t piece_b = dma_piece_b(lane, i & 1);
+        const bool real = (int)((DC - 1) * 64 + (piece_b >> 1)) < a.D;
+        k_voff_n[i] = (uint32_t)(dma_row(lane) + 8 * i) * k_row_b + (real ? piece_b : 0u);
+    }
     // start of this batch entry's Q / K (head 0, row 0), and the same advanced to this wave's first
     // row.  Only the whole-tile kernel addresses through the latter: there every row it names
     // exists.  The ragged kernel works from ABSOLUTE row numbers instead (Q rows clamped to the last
@@ -279,14 +304,17 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     // pitch (once per unit): each lane clamps its row to the last real one (repeated rows carry
     // weight 0 in the column sums).  No branch: a taken branch costs a wave far more than these few
     // address instructions.
-    auto fetch_ragged_q = [&](const char *slice, uint32_t row_b, int first_row, int n_rows, int slot) {
+    auto fetch_ragged_q = [&](const char *slice, uint32_t row_b, int first_row, int n_rows, int slot, int chunk) {
         char *dst = my_ring + slot * SLOT_BYTES;
         int l = lane;
         FCS_OPAQUE_V(l);
 #pragma unroll
         for (int tt = 0; tt < NT; ++tt) {
             const uint32_t row = (uint32_t)min(first_row + tt * 8 + dma_row(l), n_rows - 1);
-            FCS_GLDS16(slice + ((size_t)row * row_b + dma_piece_b(l, tt & 1)), dst + tt * 1024);
+            const uint32_t col_b = dma_piece_b(l, tt & 1) + (uint32_t)(chunk * 128);
+            const char *src = slice + ((size_t)row * row_b + col_b);
+            if (NARROW && (int)(col_b >> 1) >= a.D) src = reinterpret_cast<const char *>(g_fused_zeros);  // channels past the head dim
+            FCS_GLDS16(src, dst + tt * 1024);
         }
     };
     // Read a ring slot back as an MFMA operand: lane (n, g) takes, for step tt, piece 2*tt + g of
@@ -417,13 +445,24 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             const int ua = j_ahead / ITEMS;
             const int j = j_ahead % ITEMS;
             if (j == 0 && PRE) fetch_pos_piece(j_ahead, slot, 0);  // the Q item of the pre-scaled variant is a plain load, not a tile
-            else if (j == 0) fetch_ragged_q(u_qhead[ua], q_row_b, u_qfirst[ua], a.Sq, slot);
+            else if (j < DC) fetch_ragged_q(u_qhead[ua], q_row_b, u_qfirst[ua], a.Sq, slot, j);
             else {
-                const char *tile = k_batch + k_off[ua] + (size_t)tile_first(j - 1) * k_row_b;
+                // key tile (j - DC) / DC, chunk (j - DC) % DC
+                const int chunk = (j - DC) % DC;
+                const char *tile = k_batch + k_off[ua] + (size_t)tile_first((j - DC) / DC) * k_row_b + chunk * 128;
+                if (NARROW && chunk == DC - 1) {
+                    char *dst = my_ring + slot * SLOT_BYTES;
 #pragma unroll
-                for (int tt = 0; tt < NT; ++tt) {
-                    FCS_OPAQUE_V(k_voff[tt % NVOFF]);
-                    fetch_piece_at(tile, k_voff[tt % NVOFF], slot, tt);
+                    for (int tt = 0; tt < NT; ++tt) {
+                        FCS_OPAQUE_V(k_voff_n[tt % (NARROW ? NT : 1)]);
+                        FCS_GLDS16(tile + k_voff_n[tt % (NARROW ? NT : 1)], dst + tt * 1024);
+                    }
+                } else {
+#pragma unroll
+                    for (int tt = 0; tt < NT; ++tt) {
+                        FCS_OPAQUE_V(k_voff[tt % NVOFF]);
+                        fetch_piece_at(tile, k_voff[tt % NVOFF], slot, tt);
+                    }
                 }
             }
         } else {
@@ -489,7 +528,8 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                      : "memory");
     };
 
-    half8 qf[NT], kf[2][NT];
+    half8 qf_c[DC][NT], kf[2][NT];
+    half8 (&qf)[NT] = qf_c[0];  // the Q operand of a 64-wide head (chunk 0 of a wider one)
     constexpr int TQ = TPW - 2;  // KEEP: the step at which the next unit's Q rows are requested
     // KEEP: key tile `tile` (wave-uniform, 0 .. TPW-1) of unit `ua` (0 current, 1 next) into ring slot `slot`
     auto fetch_key_tile = [&](int ua, int tile, int slot) {
@@ -531,8 +571,13 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
         if (PRE) {
             take_q_shared(unit & 1, qf);
         } else {
-            FCS_WAIT_VM(2 * NT);
-            take_issue(slot_of(0), qf);
+            // item i of the unit has landed once at most the NS - 1 - i items requested behind it are outstanding
+            FCS_WAIT_VM((NS - 1) * NT);
+            take_issue(slot_of(0), qf_c[0]);
+            if constexpr (DC == 2) {
+                FCS_WAIT_VM((NS - 2) * NT);
+                take_issue(slot_of(1), qf_c[1]);
+            }
         }
         // KEEP: does the next unit read another key head (then its first NS tiles are fetched during
         // this unit's last NS steps, in the first order; else they are the ones this unit leaves behind)
@@ -544,8 +589,8 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             FCS_WAIT_VM(0);
             take_issue(slot_of_step(0), kf[0]);
         } else {
-            FCS_WAIT_VM(1 * NT);
-            take_issue(slot_of(1), kf[0]);
+            FCS_WAIT_VM((NS - 1 - DC) * NT);
+            take_issue(slot_of(DC), kf[0]);
         }
         floatx16 acc[TPW];
         float rs[16];
@@ -573,14 +618,15 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                          "+v"(rs[14]), "+v"(rs[15]));
         };
 
-        // ---------------- phase 1: one step per key tile
+        // ---------------- phase 1: one step per key tile (per half tile of a 128-wide head: chunk dc of tile t)
 #pragma unroll
-        for (int t = 0; t < TPW; ++t) {
+        for (int s = 0; s < TPW * DC; ++s) {
+            const int t = s / DC, dc = s % DC;
             // The two waves that share a SIMD (w and w + 4) take turns at the higher issue priority, one
-            // key tile each.  With equal priorities the older wave wins every arbitration, finishes
+            // step each.  With equal priorities the older wave wins every arbitration, finishes
             // its tiles ~20 % early and idles at the barrier while the other one runs alone, without
             // anything to overlap its MFMAs with (measured: 2-3 % of the kernel).
-            if (((t & 1) != 0) == (wave >= 4)) asm volatile("s_setprio 2");
+            if (((s & 1) != 0) == (wave >= 4)) asm volatile("s_setprio 2");
             else asm volatile("s_setprio 0");
             // the operands of this tile were read back during the previous step: they have landed,
             // their ring slots are free again and take the look-ahead fetches
@@ -606,29 +652,33 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
                 }
                 if (t + 1 < TPW) take_issue(slot_of_step(t + 1), kf[(t + 1) & 1]);
             } else {
-            if (t == 0) {
-                take_wait(qf);
-                take_wait(kf[0]);
-                if (!PRE && a.negate) {
+            // private rings (never pre-scaled): item DC + s is this step's key (half) tile
+            if (s == 0) {
 #pragma unroll
-                    for (int tt = 0; tt < NT; ++tt) qf[tt] = flip_sign(qf[tt]);
+                for (int ch = 0; ch < DC; ++ch) take_wait(qf_c[ch]);
+                take_wait(kf[0]);
+                if (a.negate) {
+#pragma unroll
+                    for (int ch = 0; ch < DC; ++ch)
+#pragma unroll
+                        for (int tt = 0; tt < NT; ++tt) qf_c[ch][tt] = flip_sign(qf_c[ch][tt]);
                 }
-                fetch_pos(0 + NS, slot_of(0));
-                fetch_pos(1 + NS, slot_of(1));
+#pragma unroll
+                for (int i = 0; i <= DC; ++i) fetch_pos(i + NS, slot_of(i));
             } else {
-                take_wait(kf[t & 1]);
-                fetch_pos(1 + t + NS, slot_of(1 + t));
+                take_wait(kf[s & 1]);
+                fetch_pos(DC + s + NS, slot_of(DC + s));
             }
-            // the next key tile has landed; the two items fetched after it may be in flight
-            if (item_vm(t + 3) + item_vm(t + 4) == 2 * NT) FCS_WAIT_VM(2 * NT);
-            else FCS_WAIT_VM(NT + 1);
-            if (t + 1 < TPW) take_issue(slot_of(2 + t), kf[(t + 1) & 1]);
+            // the next key (half) tile has landed; the NS - 1 items fetched after it may be in flight
+            FCS_WAIT_VM((NS - 1) * NT);
+            if (s + 1 < TPW * DC) take_issue(slot_of(DC + s + 1), kf[(s + 1) & 1]);
             }
             floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            if (dc > 0) c = acc[t];  // the second chunk's products join the first's
 #pragma unroll
-            for (int tt = 0; tt < NT; ++tt) c = mfma16<BF>(qf[tt], kf[t & 1][tt], c);
+            for (int tt = 0; tt < NT; ++tt) c = mfma16<BF>(qf_c[dc][tt], kf[s & 1][tt], c);
             acc[t] = c;
-            if (t > 0) exp_tile(t - 1);  // VALU work of the previous tile runs under this tile's MFMAs
+            if (dc == DC - 1 && t > 0) exp_tile(t - 1);  // VALU work of the previous tile runs under this tile's MFMAs
         }
         exp_tile(TPW - 1);
 
@@ -680,20 +730,24 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
             const _Float16 *qp = reinterpret_cast<const _Float16 *>(q_batch + (int64_t)h * q_head_b) +
                                  (int64_t)min(q_first + n_s, a.Sq - 1) * a.qs_s + g_s * 8;
             const _Float16 *kp = reinterpret_cast<const _Float16 *>(k_batch + (int64_t)kv_head(h, a.kv_group, a.kv_magic) * k_head_b) + g_s * 8;
-            half8 qs[NT];
+            half8 qs[DC * NT];
 #pragma unroll
-            for (int tt = 0; tt < NT; ++tt) {
-                const half8 v = load8(qp + tt * 16);
+            for (int tt = 0; tt < DC * NT; ++tt) {
+                half8 v = kZero8;  // (NARROW) channels past the tensor's head dim are zeros
+                if (!NARROW || tt * 16 + g_s * 8 < a.D) v = load8(qp + tt * 16);
                 qs[tt] = a.negate ? flip_sign(v) : v;
             }
             auto score_tile = [&](int t) {
-                half8 ks[NT];
+                half8 ks[DC * NT];
                 const int krow = RAGGED ? tile_first(t) + n_s : kbase + t * 32 + n_s;
 #pragma unroll
-                for (int tt = 0; tt < NT; ++tt) ks[tt] = load8(kp + (int64_t)krow * a.ks_s + tt * 16);
+                for (int tt = 0; tt < DC * NT; ++tt) {
+                    ks[tt] = kZero8;
+                    if (!NARROW || tt * 16 + g_s * 8 < a.D) ks[tt] = load8(kp + (int64_t)krow * a.ks_s + tt * 16);
+                }
                 floatx16 c = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int tt = 0; tt < NT; ++tt) c = mfma16<BF>(qs[tt], ks[tt], c);
+                for (int tt = 0; tt < DC * NT; ++tt) c = mfma16<BF>(qs[tt], ks[tt], c);
                 return c;
             };
             float v16[16];
@@ -774,6 +828,9 @@ struct FusedVariant {
 static FusedVariant pick_fused(const Plan &p, const Args &a, bool bf)
 {
     const int TPW = p.f_tpw;
+    // head dims other than 64: the ragged private-ring variant (two chunks per tile above 64 channels; channels past
+    // the head dim read as zeros)
+    if (p.D != 64) return {TPW, true, 0, true};
     const bool whole = p.Sk == p.f_kg * TPW * 32 && p.Sq % (32 * p.f_qg) == 0 && a.qs_s == 64 && a.ks_s == 64;
     // shared-Q variants: five to eight tiles per wave and 8, 4 or 2 key groups (S 257 .. 2048)
     const bool shared_q = TPW >= 5 && (p.f_kg == 8 || p.f_kg == 4 || p.f_kg == 2);
@@ -794,7 +851,13 @@ static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
     const dim3 grid(p.f_nwgq * p.B, p.f_hg);  // x = batch entry * f_nwgq + workgroup along the query axis
     constexpr int TPWS = (TPW >= 5) ? TPW : 8;
     const FusedVariant v = pick_fused(p, a, BF);
-    if (v.pre == 8 && v.qs && !v.ragged)
+    if (p.Dp == 128 && p.D == 128)
+        hipLaunchKernelGGL((fcs_fused_kernel<128, TPW, true, 0, BF>), grid, dim3(512), 0, st, a);
+    else if (p.Dp == 128)
+        hipLaunchKernelGGL((fcs_fused_kernel<128, TPW, true, 0, BF, true, true>), grid, dim3(512), 0, st, a);
+    else if (p.D != 64)
+        hipLaunchKernelGGL((fcs_fused_kernel<64, TPW, true, 0, BF, true, true>), grid, dim3(512), 0, st, a);
+    else if (v.pre == 8 && v.qs && !v.ragged)
         hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 8, false>), grid, dim3(512), 0, st, a);
     else if (v.pre == 4 && v.qs && !v.ragged)
         hipLaunchKernelGGL((fcs_fused_kernel<64, 8, false, 4, false>), grid, dim3(512), 0, st, a);
@@ -817,8 +880,9 @@ static void launch_tpw(const Plan &p, const Args &a, hipStream_t st)
 size_t describe_fused(const Plan &p, const Args &a, char *buf, size_t n)
 {
     const FusedVariant v = pick_fused(p, a, p.bf16 != 0);
-    int r = snprintf(buf, n, "fcs_fused_kernel<64,%d,%s,%d,%s,%s> grid %d x %d, %d x %d units per workgroup, %d slabs", v.tpw,
+    int r = snprintf(buf, n, "fcs_fused_kernel<%d,%d,%s,%d,%s,%s%s> grid %d x %d, %d x %d units per workgroup, %d slabs", p.Dp == 128 ? 128 : 64, v.tpw,
                      v.ragged ? "true" : "false", v.pre, (p.bf16 && !(v.pre && v.qs)) ? "true" : "false", v.qs ? "true" : "false",
+                     (p.D % 64 != 0) ? ",true" : "",
                      p.f_nwgq * p.B, p.f_hg, p.f_hpg, p.f_rbpw, p.n_partials);
     if (r < 0) return 0;
     const size_t len = (size_t)r;

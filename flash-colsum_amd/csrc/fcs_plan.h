@@ -232,11 +232,16 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
     // ---- fused path
     p.n_partials = p.c_groups;
     // (at least one whole key tile: the kernel moves a tile that reaches past the last key back to end there)
-    if (!causal && Sk >= 32 && Sk <= kFusedMaxKeys && D == 64) {
+    // (64-wide kernels for head dims up to 64, 128-wide ones up to 128; wider heads take the two-pass path)
+    // (Heads of 72 .. 120 channels: the 128-wide kernel's variant for narrower heads runs out of registers at seven
+    // and eight key tiles per wave, so it takes at most six, i.e. 1536 keys; longer calls take the two-pass path.)
+    const bool narrow128 = D > 64 && D < 128;
+    if (!causal && Sk >= 32 && Sk <= (narrow128 ? 8 * 6 * 32 : kFusedMaxKeys) && D <= 128) {
         p.fused = 1;
         const int tiles = ceil_div(Sk, 32);
         p.f_kg = 1;
         while (p.f_kg * 8 < tiles) p.f_kg *= 2;  // <= 8 tiles per wave
+        if (narrow128) while (p.f_kg * 6 < tiles) p.f_kg *= 2;  // <= 6 there
         p.f_qg = 8 / p.f_kg;
         p.f_tpw = ceil_div(tiles, p.f_kg);
         p.f_nqblk = ceil_div(p.q_rows, 32 * p.f_qg);
@@ -267,7 +272,7 @@ inline bool make_plan(Plan &p, int causal, int B, int H, int Sq, int Sk, int D, 
                 // the same time outgrow the XCD's 4 MiB L2, the re-reads of a head's keys by its row
                 // blocks miss (measured +6 % at B 256, S 1024 with 32 batch entries per XCD).
                 const long streams = (nwgq >= 32) ? 1 : (32 + nwgq - 1) / nwgq;
-                if (streams * (long)Sk * 128 > (5L << 19)) cost *= 1.08;
+                if (streams * (long)Sk * (2 * p.Dp) > (5L << 19)) cost *= 1.08;
                 if (first || cost < best) {
                     first = false;
                     best = cost;

@@ -431,6 +431,48 @@ def test_other_head_dims(d):
         _assert_close(out, _oracle(q, k, is_causal=True, scale=0.05), f"C ABI D={d}")
 
 
+@pytest.mark.parametrize("shape,kw,bf16,boost", [
+    ((8, 16, 1024, 128), {}, False, 0.0),                 # 128-wide heads, eight tiles x four key groups
+    ((2, 4, 2048, 128), {"scale": -0.0884}, False, 0.0),  # eight key groups, the sign on the Q chunks
+    ((3, 5, 333, 128), {}, True, 0.0),                    # ragged, bf16, two key groups
+    ((2, 3, 1500, 128), {"cls_len": 700}, False, 0.0),    # six tiles per wave (static ring slots)
+    ((2, 6, 1792, 128), {}, False, 0.0),                  # seven tiles per wave
+    ((4, 4, 100, 128), {}, False, 0.0),                   # one key group, four tiles
+    ((4, 8, 577, 80), {}, False, 0.0),                    # ViT-H: 80 channels, the upper chunk's last 48 read as zeros
+    ((2, 8, 730, 72), {}, True, 0.0),                     # SigLIP: 72 channels
+    ((2, 4, 1024, 96), {}, False, 0.0),
+    ((2, 4, 1536, 112), {"scale": 0.05}, False, 0.0),      # the longest a 72 .. 120-channel head takes on this path
+    ((2, 8, 600, 32), {}, False, 0.0),                    # narrow heads past the short-sequence kernel: 64-wide fused kernel
+    ((2, 8, 1200, 48), {}, True, 0.0),
+    ((3, 4, 300, 8), {"scale": 0.3}, False, 0.0),
+    ((2, 4, 1024, 128), {}, False, 40.0),                 # rows that leave the unstabilised range: the in-kernel exact path
+    ((2, 4, 600, 80), {}, False, 40.0),
+    ((2, 4, 600, 40), {}, True, 40.0),
+])
+def test_fused_path_for_head_dims_other_than_64(shape, kw, bf16, boost):
+    """Non-causal calls with 32 .. 2048 keys and any head dim up to 128 stay on the single-pass kernel: heads above
+    64 channels as two 64-channel chunks per operand tile, channels past the head dim as zeros.  Dense and
+    (B,S,H,D) storage give the same bits."""
+    from flash_colsum import _hip
+
+    g = torch.Generator().manual_seed(71)
+    q = torch.randn(shape, generator=g)
+    k = torch.randn(shape, generator=g)
+    if boost:
+        q[:, 1, 10:40] *= boost
+    q, k = (q.bfloat16(), k.bfloat16()) if bf16 else (q.half(), k.half())
+    text = _hip.plan_description(shape, shape, cls_n=kw.get("cls_len", -1), scale=kw.get("scale"), bf16=bf16)
+    print("fused, other head dim", shape, kw, text, flush=True)
+    assert "fcs_fused_kernel" in text
+    ref = _oracle(q.float(), k.float(), **kw)
+    out = _run(q, k, **kw)
+    _assert_close(out, ref, f"fused D={shape[3]} {shape} {kw} bf16={bf16} boost={boost}")
+    assert torch.equal(out, _run(q, k, **kw))
+    qs = q.cuda().permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)  # (B,S,H,D) storage
+    ks = k.cuda().permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    assert torch.equal(out, _run(qs, ks, **kw))
+
+
 def test_head_dims_the_library_rejects():
     with pytest.raises(RuntimeError, match="head dim"):
         _run(*_inputs((1, 2, 16, 264), (1, 2, 16, 264)))

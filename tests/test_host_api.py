@@ -205,6 +205,12 @@ def test_plan_description_and_k_past_clamp():
     assert "fcs_small_kernel<1,false,false>" in d((2, 3, 5, 40), (2, 3, 5, 40))
     assert "fcs_fused_kernel" in d((6, 24, 197, 64), (6, 24, 197, 64), cls_n=33)  # two row tiles per head: too many heads per step
     assert "fcs_fused_kernel" in d((2, 4, 289, 64), (2, 4, 289, 64))
+    # head dims other than 64 on the single-pass kernels: 128-wide ones above 64 channels, zeros past the head dim
+    assert "fcs_fused_kernel<128,8,true,0,false,true> " in d((8, 16, 1024, 128), (8, 16, 1024, 128))
+    assert "fcs_fused_kernel<128,4,true,0,false,true,true>" in d((8, 16, 1024, 96), (8, 16, 1024, 96))
+    assert "fcs_fused_kernel<64,8,true,0,true,true,true>" in d((8, 16, 2048, 32), (8, 16, 2048, 32), bf16=True)
+    assert "fcs_rowstream_kernel<128" in d((8, 16, 2048, 96), (8, 16, 2048, 96))     # 72 .. 120 channels stop at 1536 keys
+    assert "fcs_rowstream_kernel<256" in d((8, 16, 1024, 160), (8, 16, 1024, 160))
     t = d((1, 32, 512, 128), (1, 32, 65536, 128), causal=True)
     assert "fcs_rowstream_kernel<128,2,8,false,false>" in t and "fcs_colstream_kernel<128,2,8,false,false>" in t
     # 64-wide heads, 32 x 512 = 16384 averaged rows: both passes on the pre-scaled operand for the keys every row sees
