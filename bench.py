@@ -39,6 +39,9 @@ WORKLOADS = {
     "cls1_b32_h16_s577_d64": ((32, 16, 577, 64), (32, 16, 577, 64), dict(cls_len=1), False),
     # a point of the reference's own batched sweep (benchmarks/benchmark_colsum.py:289-330), not a headline config
     "noncausal_b256_h16_s1024_d64": ((256, 16, 1024, 64), (256, 16, 1024, 64), dict(), False),
+    # not in the reference's benchmarks: a vision encoder's token count (short-sequence kernel) and 128-wide heads
+    "noncausal_b64_h12_s197_d64": ((64, 12, 197, 64), (64, 12, 197, 64), dict(), False),
+    "noncausal_b8_h16_s1024_d128": ((8, 16, 1024, 128), (8, 16, 1024, 128), dict(), False),
     "causal_h32_q128_k4096_d128": ((1, 32, 128, 128), (1, 32, 4096, 128), dict(is_causal=True), False),
     "causal_h32_q128_k16384_d128": ((1, 32, 128, 128), (1, 32, 16384, 128), dict(is_causal=True), False),
     "causal_h32_q512_k65536_d128_peaky": ((1, 32, 512, 128), (1, 32, 65536, 128), dict(is_causal=True), False),

@@ -1,5 +1,6 @@
 // Attention column means on gfx950 (MI355X): fused single-kernel path for non-causal
-// calls whose whole key range fits in one workgroup's registers (32 <= S_k <= 2048, D = 64).
+// calls whose whole key range fits in one workgroup's registers (32 <= S_k <= 2048, head dims up to 128:
+// 64 channels natively, 128 as two 64-channel chunks, anything narrower on one of those two with zeros in Q).
 //
 // One workgroup = 8 waves.  The waves form a (query group) x (key group) grid; a wave
 // computes the 32 x (32 * tiles) block of scores  S = Q_tile * K_tile^T  for its 32 query
@@ -363,12 +364,12 @@ __global__ __launch_bounds__(512, 2) void fcs_fused_kernel(const Args a)
     auto tile_of = [&](int t) { return !rot ? t : KEEP_ROT ? (t + NS) % TPW : TPW - 1 - t; };
     auto slot_of_step = [&](int t) { return KEEP_ROT ? t % NS : tile_of(t) % NS; };
 
-    // The walk.  Every head contributes ITEMS = 1 + TPW operand tiles ("items"): its Q tile, then
-    // the wave's key tiles.  Item number p (counted over the whole walk) lives in ring slot p % 3.
+    // The walk.  Every head contributes ITEMS = DC * (1 + TPW) operand (half) tiles ("items"): its Q tile, then
+    // the wave's key tiles, chunk by chunk.  Item number p (counted over the whole walk) lives in ring slot p % NS.
     //   * Items are read back into registers ONE STEP BEFORE the MFMAs that use them, so the LDS
     //     latency is covered by the exponent work of the step in between.
-    //   * As soon as the read-back of item p has landed its slot is free, and item p + 3 is
-    //     fetched into it; at most three items (12 DMA instructions) are in flight.
+    //   * As soon as the read-back of item p has landed its slot is free, and item p + NS is
+    //     fetched into it; at most NS items (4 * NS DMA instructions) are in flight.
     //   * Past the last head the fetches repeat it, so that the number of outstanding DMA
     //     instructions at every wait is a compile-time constant.
     // PRE: the Q item of a head is not a tile in the ring but this wave's 32 / PRE rows of its query
