@@ -42,6 +42,12 @@ WORKLOADS = {
     # not in the reference's benchmarks: a vision encoder's token count (short-sequence kernel) and 128-wide heads
     "noncausal_b64_h12_s197_d64": ((64, 12, 197, 64), (64, 12, 197, 64), dict(), False),
     "noncausal_b8_h16_s1024_d128": ((8, 16, 1024, 128), (8, 16, 1024, 128), dict(), False),
+    # further variants of the single-pass kernels, for their profiles: nine-tile short sequences, two key groups,
+    # ragged key tiles (no multiple of 32), a head dim between 64 and 128
+    "noncausal_b32_h16_s257_d64": ((32, 16, 257, 64), (32, 16, 257, 64), dict(), False),
+    "noncausal_b128_h16_s512_d64": ((128, 16, 512, 64), (128, 16, 512, 64), dict(), False),
+    "noncausal_b32_h16_s577_d64": ((32, 16, 577, 64), (32, 16, 577, 64), dict(), False),
+    "noncausal_b8_h16_s1024_d96": ((8, 16, 1024, 96), (8, 16, 1024, 96), dict(), False),
     "causal_h32_q128_k4096_d128": ((1, 32, 128, 128), (1, 32, 4096, 128), dict(is_causal=True), False),
     "causal_h32_q128_k16384_d128": ((1, 32, 128, 128), (1, 32, 16384, 128), dict(is_causal=True), False),
     "causal_h32_q512_k65536_d128_peaky": ((1, 32, 512, 128), (1, 32, 65536, 128), dict(is_causal=True), False),
@@ -112,6 +118,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16"], help="operand type (the headline is fp16)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sweep", action="store_true",
                     help="instead of the benchmark line: run the reference's three sweeps (bench_sweep.py) and write "
@@ -140,8 +147,9 @@ def main():
         return
     name = args.workload
     q32, k32, kwargs = make_inputs(name)
-    q = q32.half().cuda()
-    k = k32.half().cuda()
+    op_dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float16
+    q = q32.to(op_dtype).cuda()
+    k = k32.to(op_dtype).cuda()
     torch.cuda.synchronize()
 
     # ---- whole-call wall clock (the headline): K calls back to back between two syncs.
@@ -179,7 +187,7 @@ def main():
     out = torch.empty((b, sk), dtype=torch.float32, device="cuda")
     call.q, call.k, call.out, call.out_f16 = q.data_ptr(), k.data_ptr(), out.data_ptr(), None
     call.ws, call.ws_bytes, call.hip_stream = ws.data_ptr(), n_ws, stream
-    plan_text = _hip.plan_description(q.shape, k.shape, causal=causal, cls_n=cls_n, scale=scale)
+    plan_text = _hip.plan_description(q.shape, k.shape, causal=causal, cls_n=cls_n, scale=scale, bf16=args.dtype == "bf16")
 
     def launch():
         rc = lib.fcs_colsum_call(call_ref)
@@ -241,7 +249,7 @@ def main():
         with open(traffic_file) as f:
             measured = json.load(f)
         if measured.get("kernel_source_sha16") == kernel_source_sha16():
-            roofline["traffic"] = measured.get(name)
+            roofline["traffic"] = measured.get(name if args.dtype == "fp16" else name + "_" + args.dtype)
         else:
             roofline["traffic_note"] = "profiles/hbm_traffic.json was measured with other kernel sources: ignored"
 
@@ -250,7 +258,7 @@ def main():
     if not args.no_cpu_baseline:
         from oracle import naive_colsum
 
-        qc, kc = q32.half().float(), k32.half().float()
+        qc, kc = q32.to(op_dtype).float(), k32.to(op_dtype).float()
         naive_colsum(qc, kc, **kwargs)
         ts = []
         for _ in range(3):
@@ -284,9 +292,9 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "fp16",
-        "dtype_note": "fp16 MFMA operands, fp32 accumulation, fp32 softmax and column sums",
-        "data": "synthetic: N(0,1) from torch.Generator(seed 0) on CPU, rounded to fp16",
+        "dtype": args.dtype,
+        "dtype_note": f"{args.dtype} MFMA operands, fp32 accumulation, fp32 softmax and column sums",
+        "data": f"synthetic: N(0,1) from torch.Generator(seed 0) on CPU, rounded to {args.dtype}",
         "config": {"workload": name, "q_shape": list(q.shape), "k_shape": list(k.shape), **{k_: v for k_, v in kwargs.items()}},
         "frac_of_fp16_mfma_peak": round(tflops / PEAK_FP16_TFLOPS, 4),
         "roofline": roofline,
