@@ -328,7 +328,8 @@ __global__ __launch_bounds__(512, 2) void fcs_small_kernel(const Args a)
         // ---------------- row sums over the key lanes (in registers); w = 1/L, 0 for rows that are not averaged
         const float L = fold_lanes_sum(rs, lane);
         const bool row_real = row0 + row_w < a.q_rows;
-        const bool bad = row_real && !(L >= kSmallSumLo && L < (PRE ? kSmallSumHiPre : kSmallSumHi));
+        // a row that is not averaged carries weight 0, but its exponentials must still be finite (inf * 0 is NaN)
+        const bool bad = row_real ? !(L >= kSmallSumLo && L < (PRE ? kSmallSumHiPre : kSmallSumHi)) : !(L < kSmallSumHi);
         const bool slow = __builtin_amdgcn_ballot_w64(bad) != 0;
         if (!slow) {
             float w16[16];

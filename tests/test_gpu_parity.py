@@ -1055,6 +1055,24 @@ def test_short_sequences_single_wave_kernel(shape, d, kw, bf16, boost):
     assert torch.equal(out, _run(qs, ks, **kw))
 
 
+@pytest.mark.parametrize("shape,cls_len,scale", [((5, 3, 9, 16), 1, 4.0), ((4, 6, 197, 64), 5, None), ((2, 8, 257, 32), 40, None),
+                                                 ((2, 4, 600, 64), 7, None), ((2, 4, 700, 128), 33, None), ((1, 4, 3000, 64), 50, None)])
+def test_rows_that_are_not_averaged_may_overflow(shape, cls_len, scale):
+    """Rows past `cls_len` carry weight 0 in the column sums, but the kernels still exponentiate them when they share
+    a tile with averaged rows: exponentials that overflow there (inf * 0) must not reach the means."""
+    g = torch.Generator().manual_seed(53)
+    q = torch.randn(shape, generator=g)
+    k = torch.randn(shape, generator=g)
+    q[:, :, cls_len:] *= 60.0
+    q, k = q.half(), k.half()
+    kw = {"cls_len": cls_len}
+    if scale is not None:
+        kw["scale"] = scale
+    out = _run(q, k, **kw)
+    assert torch.isfinite(out).all()
+    _assert_close(out, _oracle(q.float(), k.float(), **kw), f"unaveraged rows overflow {shape} cls {cls_len}")
+
+
 def test_short_sequences_with_grouped_heads_and_unequal_lengths():
     """The same kernel behind flash_colsum_ext: grouped key heads, S_q != S_k."""
     from flash_colsum import flash_colsum_ext
