@@ -510,6 +510,44 @@ def test_random_shapes_every_path():
         _assert_close(_run(q, k, **kw), _oracle(q.float(), k.float(), **kw), what)
 
 
+def test_host_threads_launch_concurrently():
+    """The host layer keeps its workspaces and prepared call structs per thread: threads that launch at the same time,
+    each on a stream of its own, get the results of the single-threaded calls, bit for bit."""
+    import threading
+
+    from flash_colsum import flash_colsum, flash_colsum_f32
+
+    cases = [((2, 4, 700, 64), (2, 4, 700, 64), {}), ((1, 4, 96, 128), (1, 4, 3000, 128), {"is_causal": True}),
+             ((4, 6, 197, 64), (4, 6, 197, 64), {}), ((2, 3, 3000, 64), (2, 3, 3000, 64), {"cls_len": 2})]
+    data = []
+    for i, (qs, ks, kw) in enumerate(cases):
+        q, k = _inputs(qs, ks, seed=80 + i)
+        q, k = q.cuda(), k.cuda()
+        data.append((q, k, kw, flash_colsum_f32(q, k, **kw), flash_colsum(q, k, **kw)))
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(t):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for it in range(25):
+                    q, k, kw, want32, want16 = data[(t + it) % len(data)]
+                    got32, got16 = flash_colsum_f32(q, k, **kw), flash_colsum(q, k, **kw)
+                    stream.synchronize()
+                    if not (torch.equal(got32, want32) and torch.equal(got16, want16)):
+                        errors.append((t, it))
+        except Exception as e:  # surfaces in the main thread
+            errors.append((t, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+
+
 def test_two_streams_and_graph_replay():
     """The library keeps no mutable global state and never allocates or synchronises: calls on
     two streams may interleave, and a call can be captured into a HIP graph and replayed."""
